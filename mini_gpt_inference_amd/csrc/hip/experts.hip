@@ -1,4 +1,4 @@
-// Gated feed-forwards and experts chosen by a table.
+// Gated feed-forwards and experts chosen by a table or by a router.
 //
 // gated unit: act[n][j] = silu(z[n][j]) * z[n][F + j], z = the joint product with the gate and up
 // matrices stacked, silu(v) = v * sigmoid(v), in 32-bit.
@@ -11,6 +11,7 @@
 // then multiplies each tile by its expert's matrix; rows come from, and go to, the places that the
 // two index arrays name.  Every output element is one chain over k in order, whatever its slot.
 #include "common.h"
+#include "dtype_io.h"
 #include "launchers.h"
 
 #define EX_TILE 16
@@ -124,6 +125,96 @@ extern "C" int mgpt_gather_rows(const void* src, long ld, const int* slot_token,
   return mgpt_last_error();
 }
 
+// A router: scores of every expert for a token, in float32 whatever the rows' dtype, and the `top`
+// largest.  logit[e] = w[e] . h; score = sigmoid(logit) (kind 0) or the logit itself (kind 1);
+// chosen[n][c] is the expert with the c-th largest score (of equal scores the lower number first) and
+// weight[n][c] its score.  One workgroup a token: a wave an expert at a time, lanes along the width in a
+// fixed order, then the first wave picks the largest `top` times.
+__global__ __launch_bounds__(256) void router_topk_kernel(const void* __restrict__ h, int dtype, long ldh,
+                                                          const void* __restrict__ w, int w_dtype, const int* __restrict__ q_req,
+                                                          int width, int n_experts, int top, int kind,
+                                                          int* __restrict__ chosen, float* __restrict__ weight) {
+  __shared__ float logit[EX_MAX_EXPERTS];
+  const int n = blockIdx.x;
+  if (q_req && q_req[n] < 0) return;     // padded token
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int e = wave; e < n_experts; e += 4) {
+    float acc = 0.f;
+    for (int c = lane; c < width; c += 64)
+      acc = fmaf(load_f(w, w_dtype, (long)e * width + c), load_f(h, dtype, (long)n * ldh + c), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) logit[e] = acc;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  for (int c = 0; c < top; ++c) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < n_experts; e += 64) {
+      const float v = logit[e];
+      if (v > best) { best = v; at = e; }      // a lane's experts rise, so the lower number stays at a tie
+    }
+    const float all = wave_max(best);
+    int cand = (best == all) ? at : 0x7fffffff;
+    // the lowest number among the lanes that hold the maximum
+    for (int off = 32; off > 0; off >>= 1) {
+      const int other = __shfl_xor(cand, off);
+      cand = other < cand ? other : cand;
+    }
+    if (cand == 0x7fffffff) cand = 0;          // every score is -inf or NaN
+    if (lane == 0) {
+      chosen[(long)n * top + c] = cand;
+      weight[(long)n * top + c] = kind == 0 ? 1.0f / (1.0f + expf(-all)) : all;
+    }
+    if ((cand & 63) == lane) logit[cand] = -INFINITY;     // the lane that reads this expert takes it out
+  }
+}
+
+// h: [n_rows, ldh] rows in `dtype`; w: dense [n_experts, width] in w_dtype; chosen: int32 [n_rows, top]; weight:
+// float32 [n_rows, top].
+extern "C" int mgpt_router_topk(const void* h, int dtype, long ldh, const void* w, int w_dtype, const int* q_req, int n_rows,
+                                int width, int n_experts, int top, int kind, int* chosen, float* weight,
+                                hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!h || !w || !chosen || !weight) return MGPT_ERR_NULL;
+  if (!dtype_ok(dtype) || !dtype_ok(w_dtype)) return MGPT_ERR_BAD_DTYPE;
+  if (n_rows < 0 || width <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || top <= 0 || top > n_experts ||
+      (kind != 0 && kind != 1))
+    return MGPT_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL(router_topk_kernel, dim3(n_rows), dim3(256), 0, stream, h, dtype, ldh, w, w_dtype, q_req, width,
+                     n_experts, top, kind, chosen, weight);
+  return mgpt_last_error();
+}
+
+// sorted[s] = pair_weight[slot_pair[s]] * src[slot_token[s]] for every used slot: the rows of a step in the
+// experts' order, each scaled by its pair's weight (in float32, rounded once to the rows' dtype)
+__global__ void gather_scale_rows_kernel(const void* __restrict__ src, int dtype, long ld, const int* __restrict__ slot_token,
+                                         const int* __restrict__ slot_pair, const float* __restrict__ pair_weight,
+                                         void* __restrict__ sorted, long lds, int n_slots, int width) {
+  const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (i >= (long)n_slots * width) return;
+  const long s = i / width;
+  const int c = (int)(i - s * width);
+  const int row = slot_token[s];
+  if (row < 0) return;
+  store_f(sorted, dtype, s * lds + c, pair_weight[slot_pair[s]] * load_f(src, dtype, (long)row * ld + c));
+}
+
+extern "C" int mgpt_gather_scale_rows(const void* src, int dtype, long ld, const int* slot_token, const int* slot_pair,
+                                      const float* pair_weight, void* sorted, long lds, int n_slots, int width,
+                                      hipStream_t stream) {
+  if (n_slots == 0) return MGPT_OK;
+  if (!src || !slot_token || !slot_pair || !pair_weight || !sorted) return MGPT_ERR_NULL;
+  if (!dtype_ok(dtype)) return MGPT_ERR_BAD_DTYPE;
+  if (n_slots < 0 || width <= 0 || ld < width || lds < width) return MGPT_ERR_BAD_SHAPE;
+  const long total = (long)n_slots * width;
+  const long blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(gather_scale_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src, dtype, ld, slot_token,
+                     slot_pair, pair_weight, sorted, lds, n_slots, width);
+  return mgpt_last_error();
+}
+
 // One workgroup: counts the pairs of every expert, lays the experts' runs of slots out one after
 // the other (each padded to whole tiles), and deals the pairs into them.
 __global__ __launch_bounds__(1024) void expert_route_kernel(
@@ -141,7 +232,7 @@ __global__ __launch_bounds__(1024) void expert_route_kernel(
   for (int p = tid; p < n_pairs; p += blockDim.x) {
     const int n = p / top;
     if (q_req && q_req[n] < 0) continue;   // padded token
-    const int e = table[(long)ids[n] * top + (p - n * top)];
+    const int e = table[(long)(ids ? ids[n] : n) * top + (p - n * top)];
     if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
   }
   __syncthreads();
@@ -159,7 +250,7 @@ __global__ __launch_bounds__(1024) void expert_route_kernel(
   for (int p = tid; p < n_pairs; p += blockDim.x) {
     const int n = p / top;
     if (q_req && q_req[n] < 0) continue;
-    const int e = table[(long)ids[n] * top + (p - n * top)];
+    const int e = table[(long)(ids ? ids[n] : n) * top + (p - n * top)];
     if (e < 0 || e >= n_experts) continue;
     const int s = start[e] + atomicAdd(&count[e], 1);
     slot_token[s] = n;
@@ -168,13 +259,13 @@ __global__ __launch_bounds__(1024) void expert_route_kernel(
   }
 }
 
-// tile_rows: 16, 64 or 256 slots a tile; n_slots = n_tiles * tile_rows must hold n_rows * top pairs with
+// ids: the table's row of every token (null: the token's own number).  tile_rows: 16, 64 or 256 slots a tile; n_slots = n_tiles * tile_rows must hold n_rows * top pairs with
 // every used expert's run padded to whole tiles.  pair_slot (optional, [n_rows * top]): where each pair went.
 extern "C" int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows,
                                  int n_experts, int* slot_token, int* slot_pair, int* pair_slot, int* tile_expert,
                                  int n_slots, int n_tiles, int tile_rows, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
-  if (!ids || !table || !slot_token || !slot_pair || !tile_expert) return MGPT_ERR_NULL;
+  if (!table || !slot_token || !slot_pair || !tile_expert) return MGPT_ERR_NULL;     // ids null: row n of the table is token n's
   if (n_rows < 0 || top <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || (tile_rows != 16 && tile_rows != 64 && tile_rows != 256) || n_slots != n_tiles * tile_rows)
     return MGPT_ERR_BAD_SHAPE;
   // every expert that is used wastes less than a tile

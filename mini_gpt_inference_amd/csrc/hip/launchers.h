@@ -137,6 +137,10 @@ int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int to
     hipStream_t stream);
 int mgpt_gather_rows(const void* src, long ld, const int* slot_token, void* sorted, long lds, int n_slots, int width,
     hipStream_t stream);
+int mgpt_router_topk(const void* h, int dtype, long ldh, const void* w, int w_dtype, const int* q_req, int n_rows,
+    int width, int n_experts, int top, int kind, int* chosen, float* weight, hipStream_t stream);
+int mgpt_gather_scale_rows(const void* src, int dtype, long ld, const int* slot_token, const int* slot_pair,
+    const float* pair_weight, void* sorted, long lds, int n_slots, int width, hipStream_t stream);
 int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, const void* w, long w_stride, const int*
     tile_expert, const int* slot_token, void* out, int out_dtype, long ldo, const int* out_rows, int n_tiles,
     int tile_rows, int n_out, int k_dim, int dtype, hipStream_t stream);
@@ -151,8 +155,18 @@ int mgpt_rms_norm(const void* x, int x_dtype, long ldx, const int* rows, const f
     int accumulate, float* zero, long ldz, int zero_width, int n_rows, int groups, int x_gstride, int o_gstride,
     int width, hipStream_t stream);
 int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, const float* g0, const float* g1, const float* g2,
-    const float* g3, int n_branches, float coef, float* x, const float* gain_post, float offset, float eps, float mult,
-    const float* gain_next, void* h, int h_dtype, int n_rows, int width, hipStream_t stream);
+    const float* g3, int n_branches, float coef, int join_unit, float* x, const float* gain_post, const float* scale_post,
+    float offset, float eps, float mult, const float* gain_next, void* h, int h_dtype, int n_rows, int width,
+    hipStream_t stream);
+// gated_state.hip
+int mgpt_gated_state(const void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head, int n_group,
+    int head_dim, int value_dim, const void* a, int a_dtype, long lda, int a_off, int mode, float q_scale, float inv_tau,
+    const float* dt_bias, const float* a_log, const float* skip, float* state, long ld_state, const int* state_slots,
+    const int* cu_q, int n_req, const int* positions, float* out, long ldo, hipStream_t stream);
+// short_conv.hip
+int mgpt_short_conv(const void* u, int dtype, long ldu, int u_off, const float* w, const float* bias, int act,
+    float* state, long ld_state, const int* state_slots, const int* cu_q, const int* q_req, const int* positions,
+    int n_req, void* out, int out_dtype, long ldo, int o_off, int n_tokens, int channels, int taps, hipStream_t stream);
 // qk_prepare.hip
 int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head, int n_kv_head,
     int head_dim, int value_dim, int head_stride, const int* positions, const float* freq, int rot_dims, float norm_eps,
@@ -218,4 +232,8 @@ int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_st
   X(mgpt_rms_post_norm) \
   X(mgpt_qk_prepare) \
   X(mgpt_decay_state) \
-  X(mgpt_decay_state_chunked)
+  X(mgpt_decay_state_chunked) \
+  X(mgpt_router_topk) \
+  X(mgpt_gather_scale_rows) \
+  X(mgpt_gated_state) \
+  X(mgpt_short_conv)

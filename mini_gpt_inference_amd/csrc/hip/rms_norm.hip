@@ -2,7 +2,8 @@
 //
 //   unit(x) = x / sqrt(mean(x^2) + eps)
 //
-// rms_norm: out = [out +] mult * unit(x) * (offset + gain) [* act(gate)], per segment: a row holds
+// rms_norm: out = [out +] mult * unit(x) * (offset + gain) [* act(gate)] (or, with the gate in front of the norm,
+// unit(x * silu(gate)) in place of unit(x) and no gate behind), per segment: a row holds
 // `groups` segments of `width` values (one for a norm over the row, one per head for a norm per
 // head).  gain may be absent (a norm without a weight), offset is 1 for a gain stored as its
 // distance from one.  Rows may be gathered (`rows`), and a second buffer may be cleared on the way
@@ -10,8 +11,9 @@
 //
 // rms_post_norm: the step between two sublayers of a layer whose sublayers are normed on both
 // sides, one workgroup a row:
-//   y = sum_b coef * unit(y_b) * gain_b          (only with several branches; else y = y_0)
-//   x += mult * unit(y) * (offset + gain_post)
+//   y = sum_b coef * unit(y_b) * gain_b          (only with several branches; else y = y_0;
+//                                                 join_unit = 0: sum_b coef * y_b * gain_b, a weighted sum)
+//   x += mult * unit(y) * (offset + gain_post) (* scale_post, a scale per channel)
 //   h = unit(x) * (offset + gain_next)           (if there is a next norm)
 //   y_b = 0                                       (ready for the next sublayer's additions)
 // Sums of squares are taken in float32 in a fixed order (lane-strided, then across the wave, then
@@ -23,6 +25,7 @@
 #define RMS_ACT_NONE 0
 #define RMS_ACT_SILU 1
 #define RMS_ACT_SIGMOID 2
+#define RMS_ACT_SILU_FIRST 3      // the input is multiplied by silu(gate) before its root mean square is taken
 
 __device__ __forceinline__ float rms_gate_act(float g, int act) {
   if (act == RMS_ACT_SILU) return g / (1.0f + expf(-g));
@@ -57,30 +60,36 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
   const int src = rows ? rows[row] : row;
   const long xb = (long)src * ldx + (long)g * x_gstride;
   const int step = blockDim.x;
+  const long ob = (long)row * ldo + (long)g * o_gstride;
+  const long gb = (long)row * ldg + (long)g * o_gstride;
+  const bool gate_first = gate && gate_act == RMS_ACT_SILU_FIRST;
+  auto input = [&](int c) {
+    float v = load_f(x, x_dtype, xb + c);
+    if (gate_first) v *= rms_gate_act(load_f(gate, gate_dtype, gb + c), RMS_ACT_SILU);
+    return v;
+  };
   float xv[PT > 0 ? PT : 1];
   float ss = 0.f;
   if (PT > 0) {
 #pragma unroll
     for (int u = 0; u < PT; ++u) {
       const int c = threadIdx.x + u * step;
-      xv[u] = c < width ? load_f(x, x_dtype, xb + c) : 0.f;
+      xv[u] = c < width ? input(c) : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < PT; ++u) ss = fmaf(xv[u], xv[u], ss);
   } else {
     for (int c = threadIdx.x; c < width; c += step) {
-      const float v = load_f(x, x_dtype, xb + c);
+      const float v = input(c);
       ss = fmaf(v, v, ss);
     }
   }
   ss = block_sum(ss, scratch);
   const float r = mult / sqrtf(ss / (float)width + eps);
-  const long ob = (long)row * ldo + (long)g * o_gstride;
-  const long gb = (long)row * ldg + (long)g * o_gstride;
   auto finish = [&](int c, float v) {
     v *= r;
     if (gain) v *= offset + gain[(long)g * width + c];
-    if (gate) v *= rms_gate_act(load_f(gate, gate_dtype, gb + c), gate_act);
+    if (gate && !gate_first) v *= rms_gate_act(load_f(gate, gate_dtype, gb + c), gate_act);
     if (accumulate) v += load_f(out, out_dtype, ob + c);
     store_f(out, out_dtype, ob + c, v);
   };
@@ -91,7 +100,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
       if (c < width) finish(c, xv[u]);
     }
   } else {
-    for (int c = threadIdx.x; c < width; c += step) finish(c, load_f(x, x_dtype, xb + c));
+    for (int c = threadIdx.x; c < width; c += step) finish(c, input(c));
   }
   if (zero && g == 0)
     for (int c = threadIdx.x; c < zero_width; c += step) zero[(long)row * ldz + c] = 0.f;
@@ -138,8 +147,9 @@ struct RmsBranches {
   const float* gain[RMS_MAX_BRANCHES];
 };
 
-__global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int n_branches, float coef, float* __restrict__ x,
-                                                            const float* __restrict__ gain_post, float offset, float eps,
+__global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int n_branches, float coef, int join_unit,
+                                                            float* __restrict__ x, const float* __restrict__ gain_post,
+                                                            const float* __restrict__ scale_post, float offset, float eps,
                                                             float mult, const float* __restrict__ gain_next,
                                                             void* __restrict__ h, int h_dtype, int n_rows, int width) {
   __shared__ float scratch[4];
@@ -153,8 +163,9 @@ __global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int 
     for (int b = 0; b < n_branches; ++b) {
       const float* yb = br.y[b] + base;
       float ss = 0.f;
-      for (int c = threadIdx.x; c < width; c += 256) ss = fmaf(yb[c], yb[c], ss);
-      r[b] = coef / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
+      if (join_unit)
+        for (int c = threadIdx.x; c < width; c += 256) ss = fmaf(yb[c], yb[c], ss);
+      r[b] = join_unit ? coef / sqrtf(block_sum_256(ss, scratch) / (float)width + eps) : coef;
     }
     for (int c = threadIdx.x; c < width; c += 256) {
       float v = 0.f;
@@ -170,7 +181,7 @@ __global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int 
   const float ry = mult / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
   float sx = 0.f;
   for (int c = threadIdx.x; c < width; c += 256) {
-    const float v = x[base + c] + y0[c] * ry * (offset + gain_post[c]);
+    const float v = x[base + c] + y0[c] * ry * (offset + gain_post[c]) * (scale_post ? scale_post[c] : 1.0f);
     x[base + c] = v;
     y0[c] = 0.f;
     sx = fmaf(v, v, sx);
@@ -185,8 +196,9 @@ __global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int 
 // the sublayers' outputs and all gains are in registers before the first sum), one trip to memory instead of
 // three or five.
 template <int PT, int NB>
-__global__ __launch_bounds__(256) void rms_post_norm_row_kernel(RmsBranches br, float coef, float* __restrict__ x,
-                                                                const float* __restrict__ gain_post, float offset, float eps,
+__global__ __launch_bounds__(256) void rms_post_norm_row_kernel(RmsBranches br, float coef, int join_unit, float* __restrict__ x,
+                                                                const float* __restrict__ gain_post,
+                                                                const float* __restrict__ scale_post, float offset, float eps,
                                                                 float mult, const float* __restrict__ gain_next,
                                                                 void* __restrict__ h, int h_dtype, int n_rows, int width) {
   __shared__ float scratch[4];
@@ -202,7 +214,7 @@ __global__ __launch_bounds__(256) void rms_post_norm_row_kernel(RmsBranches br, 
       jg[b][u] = (ok && NB > 1) ? br.gain[b][c] : 1.f;
     }
     xv[u] = ok ? x[base + c] : 0.f;
-    gp[u] = ok ? gain_post[c] : 0.f;
+    gp[u] = ok ? (offset + gain_post[c]) * (scale_post ? scale_post[c] : 1.0f) : 0.f;
     gn[u] = (ok && gain_next) ? gain_next[c] : 0.f;
   }
   if (NB > 1) {
@@ -213,7 +225,7 @@ __global__ __launch_bounds__(256) void rms_post_norm_row_kernel(RmsBranches br, 
       float ss = 0.f;
 #pragma unroll
       for (int u = 0; u < PT; ++u) ss = fmaf(yv[b][u], yv[b][u], ss);
-      r[b] = coef / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
+      r[b] = join_unit ? coef / sqrtf(block_sum_256(ss, scratch) / (float)width + eps) : coef;
     }
 #pragma unroll
     for (int u = 0; u < PT; ++u) {
@@ -231,7 +243,7 @@ __global__ __launch_bounds__(256) void rms_post_norm_row_kernel(RmsBranches br, 
 #pragma unroll
   for (int u = 0; u < PT; ++u) {
     const int c = threadIdx.x + u * 256;
-    xv[u] = xv[u] + yv[0][u] * ry * (offset + gp[u]);
+    xv[u] = xv[u] + yv[0][u] * ry * gp[u];
     if (c < width) {
       x[base + c] = xv[u];
 #pragma unroll
@@ -251,8 +263,9 @@ __global__ __launch_bounds__(256) void rms_post_norm_row_kernel(RmsBranches br, 
 // y_ptrs / gain_ptrs: n_branches device pointers each (float32 [n_rows, width] buffers; [width] gains, unused
 // with one branch).  x, y: contiguous float32 rows.
 extern "C" int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, const float* g0, const float* g1,
-                                  const float* g2, const float* g3, int n_branches, float coef, float* x,
-                                  const float* gain_post, float offset, float eps, float mult, const float* gain_next,
+                                  const float* g2, const float* g3, int n_branches, float coef, int join_unit, float* x,
+                                  const float* gain_post, const float* scale_post, float offset, float eps, float mult,
+                                  const float* gain_next,
                                   void* h, int h_dtype, int n_rows, int width, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!x || !y0 || !gain_post || (gain_next && !h)) return MGPT_ERR_NULL;
@@ -262,16 +275,16 @@ extern "C" int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, co
   for (int b = 0; b < n_branches; ++b)
     if (!br.y[b] || (n_branches > 1 && !br.gain[b])) return MGPT_ERR_NULL;
 #define RPN_ROW(PT, NB)                                                                                              \
-  hipLaunchKernelGGL((rms_post_norm_row_kernel<PT, NB>), dim3(n_rows), dim3(256), 0, stream, br, coef, x, gain_post, offset, \
-                     eps, mult, gain_next, h, h_dtype, n_rows, width)
+  hipLaunchKernelGGL((rms_post_norm_row_kernel<PT, NB>), dim3(n_rows), dim3(256), 0, stream, br, coef, join_unit, x, gain_post, \
+                     scale_post, offset, eps, mult, gain_next, h, h_dtype, n_rows, width)
   if (n_branches == 1 && width <= 256 * 4) RPN_ROW(4, 1);
   else if (n_branches == 1 && width <= 256 * 8) RPN_ROW(8, 1);
   else if (n_branches == 1 && width <= 256 * 16) RPN_ROW(16, 1);
   else if (n_branches == 2 && width <= 256 * 4) RPN_ROW(4, 2);
   else if (n_branches == 2 && width <= 256 * 8) RPN_ROW(8, 2);
   else
-    hipLaunchKernelGGL(rms_post_norm_kernel, dim3(n_rows), dim3(256), 0, stream, br, n_branches, coef, x, gain_post,
-                       offset, eps, mult, gain_next, h, h_dtype, n_rows, width);
+    hipLaunchKernelGGL(rms_post_norm_kernel, dim3(n_rows), dim3(256), 0, stream, br, n_branches, coef, join_unit, x, gain_post,
+                       scale_post, offset, eps, mult, gain_next, h, h_dtype, n_rows, width);
 #undef RPN_ROW
   return mgpt_last_error();
 }

@@ -1,0 +1,87 @@
+// A short causal convolution over time, channel by channel, for steps of any shape:
+//
+//   y_t[c] = act(sum_j w[c][j] u_(t - J + 1 + j)[c] (+ b[c])),   j = 0 .. J-1
+//
+// with zeros before a request's first token: the last tap multiplies the current token.  u are
+// columns of the step's rows (a projection's output); the J - 1 inputs that precede the step's first
+// token come from the request's slot of a float32 state pool, [J - 1][C] in the order of time, which a
+// second kernel brings up to date with the step's last inputs afterwards.  Which taps reach back
+// before position 0 is decided from the token's position, so a slot that another request used needs
+// no clearing.  The sum runs over j in order, in float32, whatever the step's shape.
+#include "common.h"
+#include "dtype_io.h"
+#include "launchers.h"
+
+#define SC_MAX_TAPS 9
+
+__global__ __launch_bounds__(256) void short_conv_kernel(
+    const void* __restrict__ u, int dtype, long ldu, int u_off, const float* __restrict__ w, const float* __restrict__ bias,
+    int act, const float* __restrict__ state, long ld_state, const int* __restrict__ state_slots,
+    const int* __restrict__ cu_q, const int* __restrict__ q_req, const int* __restrict__ positions, void* __restrict__ out,
+    int out_dtype, long ldo, int o_off, int C, int J) {
+  const int n = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int r = q_req[n];
+  if (r < 0 || c >= C) return;      // a token of the padding
+  const int start = cu_q[r], p = positions[n], slot = state_slots[r];
+  float acc = bias ? bias[c] : 0.f;
+  for (int j = 0; j < J; ++j) {
+    const int back = J - 1 - j;
+    if (p - back < 0) continue;     // before the sequence's start
+    const int s = n - back;
+    float val;
+    if (s >= start) val = load_f(u, dtype, (long)s * ldu + u_off + c);
+    else if (slot >= 0) val = state[(long)slot * ld_state + (long)((J - 1) - (start - s)) * C + c];
+    else val = 0.f;
+    acc = fmaf(w[(long)c * J + j], val, acc);
+  }
+  if (act == 1) acc = acc / (1.0f + expf(-acc));
+  store_f(out, out_dtype, (long)n * ldo + o_off + c, acc);
+}
+
+// the request's last J - 1 inputs after this step: from the step's rows, or moved up inside the state
+__global__ __launch_bounds__(256) void short_conv_state_kernel(
+    const void* __restrict__ u, int dtype, long ldu, int u_off, float* __restrict__ state, long ld_state,
+    const int* __restrict__ state_slots, const int* __restrict__ cu_q, int C, int J) {
+  const int r = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int slot = state_slots[r];
+  const int start = cu_q[r], end = cu_q[r + 1], len = end - start;
+  if (slot < 0 || len <= 0 || c >= C) return;
+  float* st = state + (long)slot * ld_state;
+  float keep[SC_MAX_TAPS - 1];
+#pragma unroll
+  for (int i = 0; i < SC_MAX_TAPS - 1; ++i) {
+    if (i < J - 1) {
+      const int s = end - (J - 1) + i;
+      if (s >= start) keep[i] = load_f(u, dtype, (long)s * ldu + u_off + c);
+      else keep[i] = st[(long)(i + len) * C + c];      // i + len < J - 1: an input of an earlier step
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < SC_MAX_TAPS - 1; ++i)
+    if (i < J - 1) st[(long)i * C + c] = keep[i];
+}
+
+// u: rows in `dtype`, the C channels at u_off; w: float32 [C][J]; bias: float32 [C] or null; act: 0 none, 1 silu.
+// state: rows of ld_state floats, (J - 1) * C of them used.  out: rows in out_dtype, the C channels at o_off
+// (not the rows of u: a token reads the inputs of the tokens before it).
+extern "C" int mgpt_short_conv(const void* u, int dtype, long ldu, int u_off, const float* w, const float* bias, int act,
+                               float* state, long ld_state, const int* state_slots, const int* cu_q, const int* q_req,
+                               const int* positions, int n_req, void* out, int out_dtype, long ldo, int o_off,
+                               int n_tokens, int channels, int taps, hipStream_t stream) {
+  if (n_tokens == 0 || n_req == 0) return MGPT_OK;
+  if (!u || !w || !state || !state_slots || !cu_q || !q_req || !positions || !out) return MGPT_ERR_NULL;
+  if (!dtype_ok(dtype) || !dtype_ok(out_dtype)) return MGPT_ERR_BAD_DTYPE;
+  if (n_tokens < 0 || n_req < 0 || channels <= 0 || taps < 1 || taps > SC_MAX_TAPS || (act != 0 && act != 1) ||
+      ld_state < (long)(taps - 1) * channels || u == out)
+    return MGPT_ERR_BAD_SHAPE;
+  const int cb = (channels + 255) / 256;
+  if (cb > 65535) return MGPT_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(short_conv_kernel, dim3(n_tokens, cb), dim3(256), 0, stream, u, dtype, ldu, u_off, w, bias, act, state,
+                     ld_state, state_slots, cu_q, q_req, positions, out, out_dtype, ldo, o_off, channels, taps);
+  if (taps > 1)
+    hipLaunchKernelGGL(short_conv_state_kernel, dim3(n_req, cb), dim3(256), 0, stream, u, dtype, ldu, u_off, state, ld_state,
+                       state_slots, cu_q, channels, taps);
+  return mgpt_last_error();
+}

@@ -1121,10 +1121,11 @@ def expert_slots(n_rows: int, top: int, n_experts: int, tile: int) -> int:
     return -(-worst // tile) * tile
 
 
-def expert_route(ids: torch.Tensor, q_req: Optional[torch.Tensor], table: torch.Tensor, n_rows: int, n_experts: int,
+def expert_route(ids: Optional[torch.Tensor], q_req: Optional[torch.Tensor], table: torch.Tensor, n_rows: int, n_experts: int,
                  slot_token: torch.Tensor, slot_pair: torch.Tensor, tile_expert: torch.Tensor, tile: int,
                  pair_slot: Optional[torch.Tensor] = None) -> None:
-    """Sorts the (token, choice) pairs by expert into slots; see csrc/hip/experts.hip.  pair_slot
+    """Sorts the (token, choice) pairs by expert into slots; see csrc/hip/experts.hip.  Token n's experts are
+    row ids[n] of the table, or row n with ids None (a table made for this step, as a router's).  pair_slot
     ([n_rows * top], optional) receives the slot of every pair."""
     _need_cuda(ids, q_req, table, slot_token, slot_pair, tile_expert, pair_slot)
     _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "the table must be dense int32")
@@ -1132,7 +1133,10 @@ def expert_route(ids: torch.Tensor, q_req: Optional[torch.Tensor], table: torch.
     top = table.shape[1]
     n_slots = expert_slots(n_rows, top, n_experts, tile)
     _need(n_experts <= MAX_EXPERTS, f"the route kernel takes up to {MAX_EXPERTS} experts")
-    _need_i32("ids", ids, n_rows)
+    if ids is not None:
+        _need_i32("ids", ids, n_rows)
+    else:
+        _need(table.shape[0] >= n_rows, "a table without ids has a row per token")
     if q_req is not None:
         _need_i32("q_req", q_req, n_rows)
     _need_i32("slot_token", slot_token, n_slots)
@@ -1217,6 +1221,49 @@ def gather_rows(src: torch.Tensor, slot_token: torch.Tensor, out: torch.Tensor, 
     return True
 
 
+ROUTER_SCORES = {"sigmoid": 0, "logit": 1}
+
+
+def router_topk(h: torch.Tensor, w: torch.Tensor, n_rows: int, top: int, chosen: torch.Tensor, weight: torch.Tensor,
+                q_req: Optional[torch.Tensor] = None, score: str = "sigmoid") -> None:
+    """chosen[n] = the `top` experts with the largest w[e] . h[n] (float32 sums), best first; weight[n] = their
+    scores (sigmoid of the sum, or the sum itself).  w: dense [experts, width]; chosen int32 and weight float32,
+    dense [>= n_rows, top]."""
+    _need_cuda(h, w, chosen, weight, q_req)
+    _need(score in ROUTER_SCORES, f"router score {score!r} is none of {sorted(ROUTER_SCORES)}")
+    _need(w.dim() == 2 and w.is_contiguous() and w.dtype in (torch.float32, torch.bfloat16), "the router's matrix must be dense")
+    n_experts, width = w.shape
+    _need(0 < top <= n_experts <= MAX_EXPERTS, f"top {top} of {n_experts} experts: need 0 < top <= experts <= {MAX_EXPERTS}")
+    _rows_2d("router rows", h, n_rows)
+    _need(h.shape[1] >= width, "the router's rows are narrower than its matrix")
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and chosen.dim() == 2 and chosen.shape[1] == top
+          and chosen.shape[0] >= n_rows, "chosen must be dense int32 [>= n_rows, top]")
+    _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.shape == chosen.shape,
+          "weight must be float32, shaped like chosen")
+    if q_req is not None:
+        _need_i32("q_req", q_req, n_rows)
+    rc = library.kernels().mgpt_router_topk(_ptr(h), _dtype_code(h), h.stride(0), _ptr(w), _dtype_code(w), _ptr(q_req), n_rows,
+                                            width, n_experts, top, ROUTER_SCORES[score], _ptr(chosen), _ptr(weight), _stream())
+    _check(rc, "router_topk")
+
+
+def gather_scale_rows(src: torch.Tensor, slot_token: torch.Tensor, slot_pair: torch.Tensor, pair_weight: torch.Tensor,
+                      out: torch.Tensor, n_slots: int) -> None:
+    """out[s] = pair_weight[slot_pair[s]] * src[slot_token[s]] for every used slot s < n_slots, the product in float32,
+    rounded to the rows' dtype."""
+    _need_cuda(src, slot_token, slot_pair, pair_weight, out)
+    width = src.shape[1]
+    _need(src.dim() == 2 and src.stride(1) == 1 and src.dtype in (torch.float32, torch.bfloat16), "rows must be float32 or bfloat16")
+    _need(out.dtype == src.dtype and out.dim() == 2 and out.shape[1] == width and out.shape[0] >= n_slots
+          and out.stride(1) == 1, "out must be [>= n_slots, width] like src")
+    _need(pair_weight.dtype == torch.float32 and pair_weight.is_contiguous(), "pair weights must be dense float32")
+    _need_i32("slot_token", slot_token, n_slots)
+    _need_i32("slot_pair", slot_pair, n_slots)
+    rc = library.kernels().mgpt_gather_scale_rows(_ptr(src), _dtype_code(src), src.stride(0), _ptr(slot_token), _ptr(slot_pair),
+                                                  _ptr(pair_weight), _ptr(out), out.stride(0), n_slots, width, _stream())
+    _check(rc, "gather_scale_rows")
+
+
 def grouped_linear_tiled(a: torch.Tensor, w: torch.Tensor, tile_expert: torch.Tensor, slot_token: torch.Tensor,
                          out: torch.Tensor, n_slots: int) -> bool:
     """out[s] = a[s] @ w[expert of s's tile of 256].T for the slots of every tile in use, through the
@@ -1243,7 +1290,7 @@ def grouped_linear_tiled(a: torch.Tensor, w: torch.Tensor, tile_expert: torch.Te
 
 
 # ---------------------------------------------------------------- root-mean-square norms, rotation, decaying state
-RMS_GATES = {None: 0, "silu": 1, "sigmoid": 2}
+RMS_GATES = {None: 0, "silu": 1, "sigmoid": 2, "silu_first": 3}
 
 
 def _rows_2d(name: str, t: torch.Tensor, n_rows: int) -> None:
@@ -1257,8 +1304,9 @@ def rms_norm(x: torch.Tensor, gain: Optional[torch.Tensor], out: torch.Tensor, n
              gate: Optional[torch.Tensor] = None, gate_act: Optional[str] = None, accumulate: bool = False,
              zero: Optional[torch.Tensor] = None) -> None:
     """out[i, g] = (out[i, g] +) mult * x[r, g] / sqrt(mean(x[r, g]^2) + eps) * (offset + gain[g]) (* act(gate[i, g]))
-    with r = rows[i] or i; a row holds `groups` segments of `width` values, x_group_stride / out_group_stride
-    apart (default: width).  gain: float32 [groups * width] or None.  gate: laid out like out.  zero: float32 rows
+    with r = rows[i] or i; with gate_act "silu_first" the gate acts in front of the norm instead: x * silu(gate)
+    takes x's place and nothing follows the gain.  A row holds `groups` segments of `width` values,
+    x_group_stride / out_group_stride apart (default: width).  gain: float32 [groups * width] or None.  gate: laid out like out.  zero: float32 rows
     that are cleared on the way (row i for every i)."""
     _need_cuda(x, gain, out, rows, gate, zero)
     xs = width if x_group_stride is None else int(x_group_stride)
@@ -1294,9 +1342,11 @@ MAX_NORM_BRANCHES = 4
 
 
 def rms_post_norm(branches, x: torch.Tensor, gain_post: torch.Tensor, n_rows: int, eps: float, offset: float,
-                  mult: float, gain_next: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None) -> None:
+                  mult: float, gain_next: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
+                  join_unit: bool = True, scale_post: Optional[torch.Tensor] = None) -> None:
     """branches: [(y float32 [rows, width], gain float32 [width] or None), ...].  With several branches
-    y = mean_b unit(y_b) * gain_b, else y = y_0; x += mult * unit(y) * (offset + gain_post); with gain_next
+    y = mean_b unit(y_b) * gain_b (join_unit False: y = sum_b y_b * gain_b, a weighted sum), else y = y_0;
+    x += mult * unit(y) * (offset + gain_post) (* scale_post, float32 [width]); with gain_next
     h = unit(x) * (offset + gain_next); every y_b is cleared.  unit(v) = v / sqrt(mean(v^2) + eps)."""
     nb = len(branches)
     _need(1 <= nb <= MAX_NORM_BRANCHES, f"rms_post_norm takes 1 to {MAX_NORM_BRANCHES} branches")
@@ -1313,15 +1363,16 @@ def rms_post_norm(branches, x: torch.Tensor, gain_post: torch.Tensor, n_rows: in
         gs.append(_ptr(g) if nb > 1 else None)
     ys += [None] * (MAX_NORM_BRANCHES - nb)
     gs += [None] * (MAX_NORM_BRANCHES - nb)
-    for g in (gain_post, gain_next):
+    for g in (gain_post, gain_next, scale_post):
         _need(g is None or (g.dtype == torch.float32 and g.numel() == width and g.is_contiguous()), "rms_post_norm: gains are float32 [width]")
     _need(gain_post is not None, "rms_post_norm needs the gain of the norm behind the sublayer")
     if gain_next is not None:
         _need(h is not None and h.is_contiguous() and h.shape[1] == width and h.shape[0] >= n_rows
               and h.dtype in (torch.float32, torch.bfloat16), "rms_post_norm: h must be dense rows as wide as x")
-    _need_cuda(x, gain_post, gain_next, h)
+    _need_cuda(x, gain_post, gain_next, h, scale_post)
     rc = library.kernels().mgpt_rms_post_norm(
-        *ys, *gs, nb, 1.0 / nb, _ptr(x), _ptr(gain_post), float(offset), float(eps), float(mult), _ptr(gain_next),
+        *ys, *gs, nb, 1.0 / nb if join_unit else 1.0, int(join_unit), _ptr(x), _ptr(gain_post), _ptr(scale_post),
+        float(offset), float(eps), float(mult), _ptr(gain_next),
         _ptr(h) if gain_next is not None else None, _dtype_code(h) if gain_next is not None else 0, n_rows, width, _stream())
     _check(rc, "rms_post_norm")
 
@@ -1440,3 +1491,81 @@ def decay_state_chunked(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_h
         n_req, n_tokens, _ptr(qk), _ptr(out), out.stride(0), _stream())
     _check(rc, "decay_state_chunked", 2)
     return True
+
+
+GATED_STATE_MODES = {"channel_sigmoid": 0, "head_softplus": 1}
+
+
+def gated_state(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int, n_group: int, head_dim: int,
+                value_dim: int, a: torch.Tensor, a_off: int, mode: str, state: torch.Tensor, state_slots: torch.Tensor,
+                cu_q: torch.Tensor, n_req: int, positions: torch.Tensor, out: torch.Tensor, q_scale: float = 1.0,
+                tau: float = 1.0, dt_bias: Optional[torch.Tensor] = None, a_log: Optional[torch.Tensor] = None,
+                skip: Optional[torch.Tensor] = None) -> None:
+    """Per request and head the state S [head_dim, value_dim] (float32, in the request's slot of `state`, zero before
+    position 0) goes over the request's tokens of this step: S = diag(decay_t) S + k v^T, o = S^T q (+ skip_h v).
+    q and k (n_group groups that heads share in turn) and v (per head) are columns of z's rows.  The decay comes
+    from columns of a's rows at a_off: mode "channel_sigmoid": sigmoid(a[h][d])^(1/tau) per key channel, and q
+    times q_scale; mode "head_softplus": dt = softplus(a[h] + dt_bias[h]), decay exp(-exp(a_log[h]) dt) for the
+    whole head, and k times dt.  state: float32 rows (a view of a pool's columns will do) of heads * dim * vdim
+    values; out: float32 rows of all heads' values."""
+    _need_cuda(z, a, state, state_slots, cu_q, positions, out, dt_bias, a_log, skip)
+    _need(mode in GATED_STATE_MODES, f"gated_state: mode {mode!r} is none of {sorted(GATED_STATE_MODES)}")
+    _rows_2d("gated_state z", z, 0)
+    _rows_2d("gated_state a", a, 0)
+    _need(n_head % n_group == 0, "gated_state: heads must be a multiple of groups")
+    _need(z.shape[1] >= max(q_off, k_off) + n_group * head_dim and z.shape[1] >= v_off + n_head * value_dim,
+          "gated_state: z is too narrow")
+    _need(a.shape[1] >= a_off + (n_head * head_dim if mode == "channel_sigmoid" else n_head), "gated_state: a is too narrow")
+    _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_head * value_dim,
+          "gated_state: out must be float32 rows of all heads' values")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] == n_head * head_dim * value_dim, "gated_state: state must be float32 rows of heads * dim * vdim")
+    for name, t in (("dt_bias", dt_bias), ("a_log", a_log), ("skip", skip)):
+        _need(t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n_head),
+              f"gated_state: {name} must be float32 [heads]")
+    _need(mode != "head_softplus" or (dt_bias is not None and a_log is not None), "gated_state: this mode needs dt_bias and a_log")
+    _need(0 < head_dim <= 256 and 0 < value_dim <= 256 and tau > 0.0, "gated_state takes head sizes up to 256")
+    _need_i32("state_slots", state_slots, n_req)
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need(positions.dtype == torch.int32 and positions.is_contiguous(), "positions must be int32")
+    rc = library.kernels().mgpt_gated_state(
+        _ptr(z), _dtype_code(z), z.stride(0), q_off, k_off, v_off, n_head, n_group, head_dim, value_dim, _ptr(a),
+        _dtype_code(a), a.stride(0), a_off, GATED_STATE_MODES[mode], float(q_scale), 1.0 / float(tau), _ptr(dt_bias),
+        _ptr(a_log), _ptr(skip), _ptr(state), state.stride(0), _ptr(state_slots), _ptr(cu_q), n_req, _ptr(positions),
+        _ptr(out), out.stride(0), _stream())
+    _check(rc, "gated_state")
+
+
+MAX_CONV_TAPS = 9
+CONV_ACTIVATIONS = {None: 0, "silu": 1}
+
+
+def short_conv(u: torch.Tensor, u_off: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+               state_slots: torch.Tensor, cu_q: torch.Tensor, q_req: torch.Tensor, positions: torch.Tensor, n_req: int,
+               out: torch.Tensor, o_off: int, n_tokens: int, activation: Optional[str] = None) -> None:
+    """out[t][o_off + c] = act(sum_j weight[c][j] * u_(t - taps + 1 + j)[u_off + c] (+ bias[c])) over time inside each
+    request, zeros before position 0; the taps - 1 inputs before the step's first token come from the request's
+    slot of `state` (float32 rows holding [taps - 1][channels], a view of a pool's columns will do), which is then
+    brought up to date.  weight: float32 [channels, taps]."""
+    _need_cuda(u, weight, bias, state, state_slots, cu_q, q_req, positions, out)
+    _need(activation in CONV_ACTIVATIONS, f"short_conv: activation {activation!r} is none of {sorted(map(str, CONV_ACTIVATIONS))}")
+    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.is_contiguous(), "short_conv: weight must be dense float32 [channels, taps]")
+    channels, taps = weight.shape
+    _need(1 <= taps <= MAX_CONV_TAPS, f"short_conv takes 1 to {MAX_CONV_TAPS} taps")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == channels),
+          "short_conv: bias must be float32 [channels]")
+    _rows_2d("short_conv input", u, n_tokens)
+    _rows_2d("short_conv output", out, n_tokens)
+    _need(u.shape[1] >= u_off + channels and out.shape[1] >= o_off + channels, "short_conv: rows are too narrow")
+    _need(u.data_ptr() != out.data_ptr(), "short_conv: the output cannot be the input's buffer")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= (taps - 1) * channels, "short_conv: state must be float32 rows of (taps - 1) * channels")
+    _need_i32("state_slots", state_slots, n_req)
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need_i32("q_req", q_req, n_tokens)
+    _need_i32("positions", positions, n_tokens)
+    rc = library.kernels().mgpt_short_conv(
+        _ptr(u), _dtype_code(u), u.stride(0), u_off, _ptr(weight), _ptr(bias), CONV_ACTIVATIONS[activation], _ptr(state),
+        state.stride(0), _ptr(state_slots), _ptr(cu_q), _ptr(q_req), _ptr(positions), n_req, _ptr(out), _dtype_code(out),
+        out.stride(0), o_off, n_tokens, channels, taps, _stream())
+    _check(rc, "short_conv", 2 if taps > 1 else 1)

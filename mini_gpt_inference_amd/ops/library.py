@@ -161,7 +161,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_gated_unit": [P, L, P, L, I, I, I, I, I, P],
         # root-mean-square norms, rotation and the rest in front of attention, decaying state
         "mgpt_rms_norm": [P, I, L, P, P, F, F, F, P, I, L, I, P, I, L, I, P, L, I, I, I, I, I, I, P],
-        "mgpt_rms_post_norm": [P, P, P, P, P, P, P, P, I, F, P, P, F, F, F, P, P, I, I, I, P],
+        "mgpt_rms_post_norm": [P, P, P, P, P, P, P, P, I, F, I, P, P, P, F, F, F, P, P, I, I, I, P],
         "mgpt_qk_prepare": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, L, I, P, P, P, I, I, P],
         "mgpt_decay_state": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, F, P, I, L, P],
         "mgpt_decay_state_chunked": [P, I, L, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, I, P, P, L, P],
@@ -171,6 +171,11 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_grouped_linear": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, I, I, P],
         "mgpt_grouped_linear_mfma": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, P],
         "mgpt_expert_combine": [P, P, P, P, I, I, I, F, P],
+        "mgpt_router_topk": [P, I, L, P, I, P, I, I, I, I, I, P, P, P],
+        "mgpt_gather_scale_rows": [P, I, L, P, P, P, P, L, I, I, P],
+        # a state with a decay made from the token, short convolutions
+        "mgpt_gated_state": [P, I, L, I, I, I, I, I, I, I, P, I, L, I, I, F, F, P, P, P, P, L, P, P, I, P, P, L, P],
+        "mgpt_short_conv": [P, I, L, I, P, P, I, P, L, P, P, P, P, I, P, I, L, I, I, I, I, P],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name, None)

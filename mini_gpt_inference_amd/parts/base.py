@@ -29,8 +29,12 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class WeightRequest:
-    shape: Tuple[int, ...]
+    shape: Tuple[int, ...]      # -1: a size that the stored tensor gives (the part reads it when it is bound)
     role: str
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(w in (-1, s) for w, s in zip(self.shape, shape))
 
 
 @dataclass(frozen=True)
@@ -40,6 +44,8 @@ class KVNeed:
     head_dim: int
     window: int = 0   # 0: all earlier keys; w: the last w positions
     joint: bool = False   # keys and values are one tensor (a latent that both are made from): a page holds it once
+    state_numel: int = 0  # float32 values per request that the mixer keeps beside its pages (the last inputs of a
+                          # short convolution in front of its keys, say); 0: none
 
 
 @dataclass(frozen=True)
@@ -136,6 +142,7 @@ class CacheBinding:
     group: int = -1      # cache group (kv)
     index: int = -1      # pool index inside the group (kv) or state pool index (state)
     writes: bool = True  # False: the run reads a cache that an earlier run of this step wrote
+    state: int = -1      # state pool index of a mixer that keeps per-request values beside its pages (kv); -1: none
 
 
 class WorkspaceFrozen(RuntimeError):

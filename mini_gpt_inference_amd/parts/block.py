@@ -154,8 +154,11 @@ class SandwichNorm(Arrangement):
     with m = `residual_mult`; the feed-forward half is optional.  With `branches` = B > 1 the mixer is
     B mixers side by side that read the same norm1(x) (roles mixer0 .. mixer{B-1}), and what norm1b
     sees is the mean of their outputs, each first normed with a gain of its own (roles join0 ..):
-    (1 / B) * sum_b join_b(mixer_b(h)).  All norms are RMS norms (kind "rms_norm"); the norms around
-    the sublayers share one eps and one way of storing the gain, the joins have plain gains.
+    (1 / B) * sum_b join_b(mixer_b(h)); with `join_weights` = (c_0, .., c_(B-1)) it is the weighted sum
+    sum_b c_b mixer_b(h) instead, and there are no join norms.  With `layer_scale` each sublayer's normed
+    output is multiplied channel by channel by a vector of the layer's own (`scale1`, `scale2`) before
+    it is added.  All norms are RMS norms (kind "rms_norm"); the norms around the sublayers share one
+    eps and one way of storing the gain, the joins have plain gains.
 
     The sublayers are the framework's ordinary parts: they add their output into a cleared float32
     buffer.  One kernel stands between two sublayers: it joins the branches, norms the sum, adds it
@@ -164,20 +167,55 @@ class SandwichNorm(Arrangement):
     graph_safe = True
     plan_safe = True
 
-    def __init__(self, width: int, residual_mult: float = 1.0, feed_forward: bool = True, branches: int = 1) -> None:
+    def __init__(self, width: int, residual_mult: float = 1.0, feed_forward: bool = True, branches: int = 1,
+                 join_weights=None, layer_scale: bool = False) -> None:
         self.width, self.mult = int(width), float(residual_mult)
         self.has_feed_forward, self.branches = bool(feed_forward), int(branches)
         if not 1 <= self.branches <= kernels.MAX_NORM_BRANCHES:
             raise ValueError(f"{self.branches} parallel mixers: the kernels take 1 to {kernels.MAX_NORM_BRANCHES}")
+        self.join_weights = None if join_weights is None else tuple(float(c) for c in join_weights)
+        if self.join_weights is not None and (self.branches < 2 or len(self.join_weights) != self.branches):
+            raise ValueError("join_weights gives one weight per parallel mixer")
+        self.has_layer_scale = bool(layer_scale)
         if self.branches == 1:
             self.mixer_roles, self.join_roles = ("mixer",), ()
         else:
             self.mixer_roles = tuple(f"mixer{b}" for b in range(self.branches))
-            self.join_roles = tuple(f"join{b}" for b in range(self.branches))
+            self.join_roles = () if self.join_weights is not None else tuple(f"join{b}" for b in range(self.branches))
         self.roles = ("norm1",) + self.mixer_roles + self.join_roles + ("norm1b",)
         if self.has_feed_forward:
             self.roles += ("norm2", "feed_forward", "norm2b")
         self._checked = False
+        self.scale1 = self.scale2 = None
+        self._join_gains = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        if not self.has_layer_scale:
+            return {}
+        req = {"scale1": WeightRequest((self.width,), VECTOR)}
+        if self.has_feed_forward:
+            req["scale2"] = WeightRequest((self.width,), VECTOR)
+        return req
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        first = next(iter(tensors.values()), None)
+        if first is not None and self.join_weights is not None:      # made here, not inside a step
+            self._join_gains = [torch.full((self.width,), c, dtype=torch.float32, device=first.device)
+                                for c in self.join_weights]
+        return None
+
+    def _joins(self, ys, parts):
+        """Per branch: its buffer and the vector that multiplies it in the join (a join norm's gain, or the
+        branch's constant weight on every channel)."""
+        if self.branches == 1:
+            return [(ys[0], None)]
+        if self.join_weights is None:
+            return [(ys[b], parts[self.join_roles[b]].weight) for b in range(self.branches)]
+        if self._join_gains is None or self._join_gains[0].device != ys.device:
+            self._join_gains = [torch.full((self.width,), c, dtype=torch.float32, device=ys.device)
+                                for c in self.join_weights]
+        return [(ys[b], self._join_gains[b]) for b in range(self.branches)]
 
     def _check(self, parts) -> None:
         around = [parts[r] for r in self.roles if r.startswith("norm")]
@@ -221,15 +259,16 @@ class SandwichNorm(Arrangement):
             norm1.forward(ctx, x, h, n)
         for b, role in enumerate(self.mixer_roles):
             parts[role].forward_add(ctx, h, ys[b], bindings[role], position)
-        joins = [(ys[b], parts[self.join_roles[b]].weight if B > 1 else None) for b in range(B)]
+        joins = self._joins(ys, parts)
+        join_unit = self.join_weights is None
         if not self.has_feed_forward:
-            ctx.pending_update = PendingSandwich(joins, x, parts["norm1b"], self.mult, n)
+            ctx.pending_update = PendingSandwich(joins, x, parts["norm1b"], self.mult, n, join_unit, self.scale1)
             return
         norm1b = parts["norm1b"]
         kernels.rms_post_norm(joins, x, norm1b.weight, n, norm1b.eps, norm1b.offset, self.mult,
-                              gain_next=parts["norm2"].weight, h=h)
+                              gain_next=parts["norm2"].weight, h=h, join_unit=join_unit, scale_post=self.scale1)
         parts["feed_forward"].forward_add(ctx, h, ys[0])
-        ctx.pending_update = PendingSandwich([(ys[0], None)], x, parts["norm2b"], self.mult, n)
+        ctx.pending_update = PendingSandwich([(ys[0], None)], x, parts["norm2b"], self.mult, n, True, self.scale2)
 
 
 class PendingSandwich:
@@ -237,8 +276,10 @@ class PendingSandwich:
     reads x next makes the addition: a layer of the same kind together with its first norm (run(gain, h) also
     leaves h = norm_next(x)), anyone else through flush_update."""
 
-    def __init__(self, joins, x: torch.Tensor, norm: Part, mult: float, n_rows: int) -> None:
+    def __init__(self, joins, x: torch.Tensor, norm: Part, mult: float, n_rows: int, join_unit: bool = True,
+                 scale: Optional[torch.Tensor] = None) -> None:
         self.joins, self.x, self.norm, self.mult, self.n_rows = joins, x, norm, mult, n_rows
+        self.join_unit, self.scale = join_unit, scale      # how several branches meet; the layer's scale per channel
 
     def goes_with(self, norm_next: Part, x: torch.Tensor, n_rows: int) -> bool:
         return (x is self.x and n_rows == self.n_rows and norm_next.eps == self.norm.eps
@@ -246,7 +287,7 @@ class PendingSandwich:
 
     def run(self, gain_next: Optional[torch.Tensor], h: Optional[torch.Tensor]) -> None:
         kernels.rms_post_norm(self.joins, self.x, self.norm.weight, self.n_rows, self.norm.eps, self.norm.offset,
-                              self.mult, gain_next=gain_next, h=h)
+                              self.mult, gain_next=gain_next, h=h, join_unit=self.join_unit, scale_post=self.scale)
 
 
 def flush_update(ctx: StepContext) -> None:

@@ -171,6 +171,9 @@ class TableExperts(FeedForward):
         self.table = tensors["table"]
         if self.table.dtype != torch.int32:
             raise ValueError("the experts' table must hold integers")
+        return self._bind_experts(tensors)
+
+    def _bind_experts(self, tensors):
         f, views = self.hidden, {}
         # [experts, 2 * hidden, width] and [experts, width, hidden]: an expert's matrices lie together
         self.in_weights = torch.stack([torch.cat([tensors[f"e{e}_gate"], tensors[f"e{e}_up"]], dim=0)
@@ -191,11 +194,17 @@ class TableExperts(FeedForward):
 
     def forward_add(self, ctx: StepContext, h, x: torch.Tensor) -> None:
         plain_residual(ctx, h, x)
-        n, ws = ctx.n_rows, ctx.workspace
         hn = as_tensor(ctx, h)
+        self._experts_add(ctx, hn, x, ctx.n_rows, ctx.token_ids, self.table, None, 1.0 / self.top)
+
+    def _experts_add(self, ctx: StepContext, hn: torch.Tensor, x: torch.Tensor, n: int, ids, table: torch.Tensor,
+                     pair_weight, combine_weight: float) -> None:
+        """x += combine_weight * sum over token n's experts (row ids[n] of the table, or row n without ids) of
+        expert(w h), w = pair_weight[n][choice] (None: 1), plus the shared expert."""
+        ws = ctx.workspace
         fast = not ctx.exact and ctx.dtype == torch.bfloat16
         if fast and n * self.top >= self.TILED_FROM_PAIRS and self.width % 16 == 0 and self.hidden % 16 == 0 \
-                and self._forward_tiled(ctx, hn, x, n):
+                and self._forward_tiled(ctx, hn, x, n, ids, table, pair_weight, combine_weight):
             return
         # tiles of 64 slots for the MFMA kernel of few rows, of 16 for the general one
         tile = 64 if fast else 16
@@ -203,10 +212,15 @@ class TableExperts(FeedForward):
         slot_token = ws.get("expert_slot_token", slots, 1, torch.int32).view(-1)
         slot_pair = ws.get("expert_slot_pair", slots, 1, torch.int32).view(-1)
         tile_expert = ws.get("expert_tile", slots // tile, 1, torch.int32).view(-1)
-        kernels.expert_route(ctx.token_ids, ctx.q_req, self.table, n, self.n_experts, slot_token, slot_pair,
-                             tile_expert, tile)
+        kernels.expert_route(ids, ctx.q_req, table, n, self.n_experts, slot_token, slot_pair, tile_expert, tile)
         z = ws.get("expert_z", slots, 2 * self.hidden, ctx.dtype)
-        kernels.grouped_linear(hn, slot_token, self.in_weights, tile_expert, slot_token, z, None, slots, tile, fast)
+        if pair_weight is None:
+            kernels.grouped_linear(hn, slot_token, self.in_weights, tile_expert, slot_token, z, None, slots, tile, fast)
+        else:
+            # the weight multiplies the expert's input: every pair's row is made first, scaled, in the experts' order
+            rows = ws.get("expert_rows", slots, self.width, ctx.dtype)
+            kernels.gather_scale_rows(hn, slot_token, slot_pair, pair_weight, rows, slots)
+            kernels.grouped_linear(rows, None, self.in_weights, tile_expert, slot_token, z, None, slots, tile, fast)
         act = ws.get("expert_act", slots, self.hidden, ctx.dtype)
         kernels.gated_unit(z, act, slots, self.hidden, fast=not ctx.exact)
         pair_out = ws.get("expert_pair_out", n * self.top, self.width, torch.float32)
@@ -214,7 +228,7 @@ class TableExperts(FeedForward):
                                tile, fast)
         if self.shared_hidden:
             _gated(ctx, hn, self.shared_in_weight, self.shared_down, x, n, self.shared_hidden)
-        kernels.expert_combine(pair_out, x, n, self.top, 1.0 / self.top, q_req=ctx.q_req)
+        kernels.expert_combine(pair_out, x, n, self.top, combine_weight, q_req=ctx.q_req)
 
     # From this many (token, choice) pairs on, the experts' products go through the tiled MFMA kernel
     # of the dense layers: the pairs' rows are copied into the experts' order first, every expert's
@@ -223,7 +237,8 @@ class TableExperts(FeedForward):
     # rows would be most of the work.
     TILED_FROM_PAIRS = 512
 
-    def _forward_tiled(self, ctx: StepContext, hn: torch.Tensor, x: torch.Tensor, n: int) -> bool:
+    def _forward_tiled(self, ctx: StepContext, hn: torch.Tensor, x: torch.Tensor, n: int, ids, table: torch.Tensor,
+                       pair_weight, combine_weight: float) -> bool:
         ws, tile = ctx.workspace, 256
         slots = kernels.expert_slots(n, self.top, self.n_experts, tile)
         slot_token = ws.get("expert_slot_token", slots, 1, torch.int32).view(-1)
@@ -231,11 +246,13 @@ class TableExperts(FeedForward):
         pair_slot = ws.get("expert_pair_slot", n * self.top, 1, torch.int32).view(-1)
         tile_expert = ws.get("expert_tile", slots // tile, 1, torch.int32).view(-1)
         sorted_rows = ws.get("expert_rows", slots, self.width, ctx.dtype)
-        if hn.stride(0) % 8 or hn.data_ptr() % 16 or sorted_rows.data_ptr() % 16:
+        if hn.stride(0) % 8 or hn.data_ptr() % 16 or sorted_rows.data_ptr() % 16 or self.width % 8:
             return False
-        kernels.expert_route(ctx.token_ids, ctx.q_req, self.table, n, self.n_experts, slot_token, slot_pair,
+        kernels.expert_route(ids, ctx.q_req, table, n, self.n_experts, slot_token, slot_pair,
                              tile_expert, tile, pair_slot=pair_slot)
-        if not kernels.gather_rows(hn, slot_token, sorted_rows, slots):
+        if pair_weight is not None:
+            kernels.gather_scale_rows(hn, slot_token, slot_pair, pair_weight, sorted_rows, slots)
+        elif not kernels.gather_rows(hn, slot_token, sorted_rows, slots):
             return False
         z = ws.get("expert_z", slots, 2 * self.hidden, ctx.dtype)
         if not kernels.grouped_linear_tiled(sorted_rows, self.in_weights, tile_expert, slot_token, z, slots):
@@ -247,5 +264,48 @@ class TableExperts(FeedForward):
             return False
         if self.shared_hidden:
             _gated(ctx, hn, self.shared_in_weight, self.shared_down, x, n, self.shared_hidden)
-        kernels.expert_combine(slot_out, x, n, self.top, 1.0 / self.top, pair_slot=pair_slot, q_req=ctx.q_req)
+        kernels.expert_combine(slot_out, x, n, self.top, combine_weight, pair_slot=pair_slot, q_req=ctx.q_req)
         return True
+
+
+@register_feed_forward("routed_experts")
+class RoutedExperts(TableExperts):
+    """A mixture of gated feed-forwards chosen by a router: scores s = sigmoid(h Wr^T), computed in
+    float32; a token uses the `top` experts with the largest scores; the output is the sum over them of
+    expert_e(s_e h), expert(u) = (silu(u Wgate^T) * (u Wup^T)) Wdown^T: the score multiplies the expert's
+    input and is not renormalised.  A shared expert (shared_hidden > 0) takes every token unweighted.
+
+    The router kernel writes the step's own table of experts and scores; from there on the experts run as
+    those chosen by a stored table do."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, hidden: int, n_experts: int, top: int, shared_hidden: int = 0,
+                 score: str = "sigmoid") -> None:
+        super().__init__(width, hidden, n_experts, top, vocab_size=0, shared_hidden=shared_hidden)
+        if score not in kernels.ROUTER_SCORES:
+            raise ValueError(f"router score {score!r} is none of {sorted(kernels.ROUTER_SCORES)}")
+        self.score = score
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        req = super().weight_requests()
+        del req["table"]
+        req["router_weight"] = WeightRequest((self.n_experts, self.width), MATRIX)
+        return req
+
+    def bind(self, tensors):
+        self.router_weight = tensors["router_weight"]
+        return self._bind_experts(tensors)
+
+    def token_matrix_elements(self) -> int:
+        return super().token_matrix_elements() + self.n_experts * self.width
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor) -> None:
+        plain_residual(ctx, h, x)
+        n, ws = ctx.n_rows, ctx.workspace
+        hn = as_tensor(ctx, h)
+        chosen = ws.get("router_chosen", n, self.top, torch.int32)
+        weight = ws.get("router_weight", n, self.top, torch.float32)
+        kernels.router_topk(hn, self.router_weight, n, self.top, chosen, weight, q_req=ctx.q_req, score=self.score)
+        self._experts_add(ctx, hn, x, n, None, chosen, weight.view(-1), 1.0)

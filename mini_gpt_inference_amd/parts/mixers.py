@@ -264,7 +264,10 @@ class GatedAttention(Mixer):
     cached is the rotated, normed key and the mixed value.  S = (q . k) * scale, capped as
     cap * tanh(S / cap) (`softcap`), softmax in float32 over the keys at positions <= the query's;
     head a's output times sigmoid(h Wg^T)_a, one number per head (`head_gate`); out = y Wo^T, added
-    into the residual.
+    into the residual.  With `conv_taps` = J > 1 the projected q, k and v pass a causal convolution over
+    time first, channel by channel (weights [channels, J], the last tap on the current token, zeros
+    before the sequence's start), whose last J - 1 inputs are kept per request beside the pages.  With
+    `window` = w > 0 a query sees only the keys at the last w positions, its own included.
 
     The cache keeps keys and values in pages of one head size, so both are laid out with
     max(D, E) channels a head (rounded up to what the bfloat16 attention kernels take), the
@@ -276,7 +279,7 @@ class GatedAttention(Mixer):
     def __init__(self, width: int, n_head: int, n_kv_head: int, head_dim: int, value_dim: int, scale: float,
                  bias: bool = False, rotary: Optional[dict] = None, qk_norm_eps: Optional[float] = None,
                  softcap: float = 0.0, head_gate: bool = False, value_mix: Optional[str] = None,
-                 share: str = "values") -> None:
+                 share: str = "values", conv_taps: int = 0, window: int = 0) -> None:
         self.width, self.n_head, self.n_kv_head = int(width), int(n_head), int(n_kv_head)
         self.head_dim, self.value_dim, self.scale = int(head_dim), int(value_dim), float(scale)
         self.has_bias, self.has_gate = bool(bias), bool(head_gate)
@@ -286,6 +289,9 @@ class GatedAttention(Mixer):
         if value_mix not in (None, "keep", "mix"):
             raise ValueError(f"value_mix {value_mix!r} is none of None, 'keep', 'mix'")
         self.value_mix, self.share = value_mix, str(share)
+        self.conv_taps, self.window = int(conv_taps or 0), int(window or 0)
+        if not 0 <= self.conv_taps <= kernels.MAX_CONV_TAPS or self.window < 0:
+            raise ValueError(f"{conv_taps} taps, window {window}: the convolution takes up to {kernels.MAX_CONV_TAPS} taps")
         if self.n_head % self.n_kv_head != 0:
             raise ValueError("n_head must be a multiple of n_kv_head")
         if self.rotation is not None and self.rotation.dims > self.head_dim:
@@ -299,12 +305,16 @@ class GatedAttention(Mixer):
         self.v_off = self.k_off + self.n_kv_head * s
         self.g_off = self.v_off + self.n_kv_head * s
         self.in_rows = -(-(self.g_off + (self.n_head if self.has_gate else 0)) // 16) * 16
-        self.in_weight = self.in_bias = self.out_padded = None
+        self.in_weight = self.in_bias = self.out_padded = self.conv_weight = None
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
         H, G, D, E, W = self.n_head, self.n_kv_head, self.head_dim, self.value_dim, self.width
         req = {"q_weight": WeightRequest((H * D, W), MATRIX), "k_weight": WeightRequest((G * D, W), MATRIX),
                "v_weight": WeightRequest((G * E, W), MATRIX), "out_weight": WeightRequest((W, H * E), MATRIX)}
+        if self.conv_taps > 1:
+            J = self.conv_taps
+            req.update(q_conv=WeightRequest((H * D, J), VECTOR), k_conv=WeightRequest((G * D, J), VECTOR),
+                       v_conv=WeightRequest((G * E, J), VECTOR))
         if self.has_bias:
             req.update(q_bias=WeightRequest((H * D,), VECTOR), k_bias=WeightRequest((G * D,), VECTOR),
                        v_bias=WeightRequest((G * E,), VECTOR))
@@ -339,6 +349,13 @@ class GatedAttention(Mixer):
                                           ("v_bias", self.v_off, G, E)):
                 bias[at:at + heads * s].view(heads, s)[:, :size].copy_(tensors[name].view(heads, size))
             self.in_bias = bias
+        if self.conv_taps > 1:
+            # the taps of the padded layout's channels (zeros for the channels a head does not have)
+            taps = torch.zeros((self.g_off, self.conv_taps), dtype=torch.float32, device=q.device)
+            for name, at, heads, size in (("q_conv", self.q_off, H, D), ("k_conv", self.k_off, G, D),
+                                          ("v_conv", self.v_off, G, E)):
+                taps[at:at + heads * s].view(heads, s, -1)[:, :size].copy_(tensors[name].view(heads, size, -1))
+            self.conv_weight = taps
         out = tensors["out_weight"]
         padded = torch.zeros((W, H * s), dtype=out.dtype, device=out.device)
         padded.view(W, H, s)[:, :, :E].copy_(out.view(W, H, E))
@@ -349,7 +366,8 @@ class GatedAttention(Mixer):
         return views
 
     def cache_need(self) -> KVNeed:
-        return KVNeed(self.n_kv_head, self.head_stride, 0)
+        return KVNeed(self.n_kv_head, self.head_stride, self.window,
+                      state_numel=(self.conv_taps - 1) * self.g_off if self.conv_taps > 1 else 0)
 
     def token_matrix_elements(self) -> int:
         return self.in_weight.numel() + self.out_padded.numel() if self.in_weight is not None else 0
@@ -362,6 +380,15 @@ class GatedAttention(Mixer):
         n, ws, s = ctx.n_rows, ctx.workspace, self.head_stride
         z = ws.get("gated_attention_in", n, self.in_rows, ctx.dtype)
         linear(ctx, h, self.in_weight, self.in_bias, z, n)
+        if self.conv_taps > 1:
+            # q, k and v through their short convolution into a second buffer (a token reads the inputs of the
+            # tokens before it); the gate's columns, if any, stay where they are
+            zc = ws.get("gated_attention_conv", n, self.in_rows, ctx.dtype)
+            kernels.short_conv(z, 0, self.conv_weight, None, ctx.state_pools[binding.state], ctx.state_slots, ctx.cu_q,
+                               ctx.q_req, ctx.positions, ctx.cu_q.numel() - 1, zc, 0, n)
+            gate_rows, z = z, zc
+        else:
+            gate_rows = z
         group = ctx.groups[binding.group]
         k_pool, v_pool = group.k_pools[binding.index], group.v_pools[binding.index]
         other, mode = None, 0
@@ -375,8 +402,8 @@ class GatedAttention(Mixer):
                            mix_mode=mode, k_pool=k_pool, v_pool=v_pool, slot_mapping=group.slot_mapping)
         y = ws.get("attn_out", n, self.n_head * s, ctx.dtype)
         # (the gate per head is applied by the attention kernel as it stores a head's output)
-        attention_ops.paged_attention(ctx, z, y, k_pool, v_pool, group, self.n_head, self.scale, 0, softcap=self.softcap,
-                                      gate=z[:, self.g_off:] if self.has_gate else None)
+        attention_ops.paged_attention(ctx, z, y, k_pool, v_pool, group, self.n_head, self.scale, self.window,
+                                      softcap=self.softcap, gate=gate_rows[:, self.g_off:] if self.has_gate else None)
         linear_add(ctx, y, self.out_padded, None, x, n)
 
 
@@ -484,4 +511,160 @@ class DecayStateMixer(Mixer):
         elif self.head_norm_eps is None:
             kernels.rms_norm(sums, self.norm_weight, y, n, self.out_norm_eps, self.v_width, gate=z[:, self.g_off:],
                              gate_act="sigmoid")
+        linear_add(ctx, y, self.out_weight, None, x, n)
+
+
+@register_mixer("gated_linear_attention")
+class GatedLinearAttention(Mixer):
+    """Linear attention whose state decays channel by channel at a rate made from the token: no softmax,
+    and instead of a cache one float32 matrix per request and head.
+
+    q = h Wq^T * q_scale, k = h Wk^T [H, D], v = h Wv^T [H, E]; u = (h Wa1^T) Wa2^T + b [H, D] through a narrow
+    middle; decay_t = sigmoid(u)^(1/tau) per key channel; S_t = diag(decay_t) S_(t-1) + k_t v_t^T,
+    o_t = S_t^T q_t per head, S zero before the first token.  Each head's o is divided by its root mean
+    square and multiplied by `norm_weight` [E] (one weight for all heads), the heads by silu(h Wg^T);
+    out = y Wo^T, added into the residual.  From the decay's logit on everything is float32 up to y."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, n_head: int, head_dim: int, value_dim: int, tau: float, norm_eps: float,
+                 decay_rank: Optional[int] = None, q_scale: Optional[float] = None) -> None:
+        self.width, self.n_head, self.head_dim, self.value_dim = int(width), int(n_head), int(head_dim), int(value_dim)
+        # the narrow middle of the decay's projection: given, or (None) whatever the stored tensors have
+        self.decay_rank = -1 if decay_rank is None else int(decay_rank)
+        self.tau, self.norm_eps = float(tau), float(norm_eps)
+        self.q_scale = self.head_dim ** -0.5 if q_scale is None else float(q_scale)
+        if not (0 < self.head_dim <= 256 and 0 < self.value_dim <= 256):
+            raise ValueError("the state kernel takes head sizes up to 256")
+        if not self.tau > 0.0 or self.decay_rank == 0 or self.decay_rank < -1:
+            raise ValueError(f"tau {tau} and decay rank {decay_rank} must be positive")
+        self.qk_width, self.v_width = self.n_head * self.head_dim, self.n_head * self.value_dim
+        self.k_off, self.v_off = self.qk_width, 2 * self.qk_width
+        self.g_off = self.v_off + self.v_width
+        self.a_off = self.g_off + self.v_width
+        self.in_weight = self.head_gain = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        W = self.width
+        return {"q_weight": WeightRequest((self.qk_width, W), MATRIX), "k_weight": WeightRequest((self.qk_width, W), MATRIX),
+                "v_weight": WeightRequest((self.v_width, W), MATRIX), "gate_weight": WeightRequest((self.v_width, W), MATRIX),
+                "decay_in_weight": WeightRequest((self.decay_rank, W), MATRIX),
+                "decay_out_weight": WeightRequest((self.qk_width, self.decay_rank), MATRIX),
+                "decay_out_bias": WeightRequest((self.qk_width,), VECTOR),
+                "norm_weight": WeightRequest((self.value_dim,), VECTOR),
+                "out_weight": WeightRequest((W, self.v_width), MATRIX)}
+
+    def token_matrix_elements(self) -> int:
+        if self.in_weight is None:
+            return 0
+        return self.in_weight.numel() + self.decay_out_weight.numel() + self.out_weight.numel()
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        if tensors["decay_in_weight"].shape[0] != tensors["decay_out_weight"].shape[1]:
+            raise ValueError("the two steps of the decay's projection do not fit each other")
+        self.decay_rank = int(tensors["decay_in_weight"].shape[0])
+        names = ["q_weight", "k_weight", "v_weight", "gate_weight", "decay_in_weight"]
+        self.in_weight = torch.cat([tensors[n] for n in names], dim=0).contiguous()
+        views, at = {}, 0
+        for n in names:
+            rows = tensors[n].shape[0]
+            views[n] = self.in_weight[at:at + rows]
+            setattr(self, n, views[n])
+            at += rows
+        self.head_gain = self.norm_weight.repeat(self.n_head).contiguous()    # the heads' one weight, head by head
+        return views
+
+    def cache_need(self) -> StateNeed:
+        return StateNeed(self.n_head * self.head_dim * self.value_dim)
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor, binding: CacheBinding,
+                    position: PositionEncoding) -> None:
+        if binding.kind != "state":
+            raise ValueError("gated linear attention needs a state pool")
+        plain_residual(ctx, h, x)
+        n, ws = ctx.n_rows, ctx.workspace
+        z = ws.get("gla_in", n, self.in_weight.shape[0], ctx.dtype)
+        linear(ctx, h, self.in_weight, None, z, n)
+        u = ws.get("gla_decay", n, self.qk_width, ctx.dtype)
+        linear(ctx, z[:, self.a_off:], self.decay_out_weight, self.decay_out_bias, u, n)
+        sums = ws.get("gla_sums", n, self.v_width, torch.float32)
+        kernels.gated_state(z, 0, self.k_off, self.v_off, self.n_head, self.n_head, self.head_dim, self.value_dim, u, 0,
+                            "channel_sigmoid", ctx.state_pools[binding.index], ctx.state_slots, ctx.cu_q,
+                            ctx.cu_q.numel() - 1, ctx.positions, sums, q_scale=self.q_scale, tau=self.tau)
+        y = ws.get("gla_out", n, self.v_width, ctx.dtype)
+        kernels.rms_norm(sums, self.head_gain, y, n, self.norm_eps, self.value_dim, groups=self.n_head,
+                         gate=z[:, self.g_off:], gate_act="silu")
+        linear_add(ctx, y, self.out_weight, None, x, n)
+
+
+@register_mixer("state_space")
+class StateSpaceMixer(Mixer):
+    """A selective state-space mixer in its scalar-decay (state-space duality) form: per head a float32
+    state [N, E] per request, whose decay and input step come from the token.
+
+    h Win^T is laid out [z: H*E | x: H*E | B: G*N | C: G*N | dt: H].  x, B and C together pass a causal
+    convolution over time, channel by channel (`conv_weight` [channels, J], bias, the last tap on the
+    current token, zeros before the sequence's start), then silu.  dt = softplus(dt + dt_bias); head a
+    (which reads B and C of group a // (H / G)): S_t = exp(-exp(A_log_a) dt) S_(t-1) + dt B_t x_t^T,
+    y_t = S_t^T C_t + D_a x_t.  The heads' y times silu(z), then divided by its root mean square in
+    `norm_groups` equal parts and multiplied by `norm_weight`; out = y Wo^T, added into the residual.
+    Kept per request: the state and the convolution's last J - 1 inputs.  Float32 from dt's softplus on up to
+    the normed y."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, n_head: int, value_dim: int, state_dim: int, n_group: int, conv_taps: int,
+                 norm_groups: int, norm_eps: float) -> None:
+        self.width, self.n_head, self.value_dim = int(width), int(n_head), int(value_dim)
+        self.state_dim, self.n_group, self.conv_taps = int(state_dim), int(n_group), int(conv_taps)
+        self.norm_groups, self.norm_eps = int(norm_groups), float(norm_eps)
+        self.inner = self.n_head * self.value_dim
+        if self.n_head % self.n_group or self.inner % self.norm_groups:
+            raise ValueError("heads must be a multiple of groups, and heads * vdim of the norm's parts")
+        if not (0 < self.state_dim <= 256 and 0 < self.value_dim <= 256):
+            raise ValueError("the state kernel takes head sizes up to 256")
+        if not 1 <= self.conv_taps <= kernels.MAX_CONV_TAPS:
+            raise ValueError(f"the convolution takes 1 to {kernels.MAX_CONV_TAPS} taps")
+        self.conv_width = self.inner + 2 * self.n_group * self.state_dim
+        self.dt_off = self.inner + self.conv_width
+        self.in_rows = self.dt_off + self.n_head
+        self.state_numel = self.n_head * self.state_dim * self.value_dim
+        self.conv_numel = (self.conv_taps - 1) * self.conv_width
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        H = self.n_head
+        return {"in_weight": WeightRequest((self.in_rows, self.width), MATRIX),
+                "conv_weight": WeightRequest((self.conv_width, self.conv_taps), VECTOR),
+                "conv_bias": WeightRequest((self.conv_width,), VECTOR),
+                "dt_bias": WeightRequest((H,), VECTOR), "a_log": WeightRequest((H,), VECTOR),
+                "skip": WeightRequest((H,), VECTOR), "norm_weight": WeightRequest((self.inner,), VECTOR),
+                "out_weight": WeightRequest((self.width, self.inner), MATRIX)}
+
+    def cache_need(self) -> StateNeed:
+        return StateNeed(self.state_numel + self.conv_numel)
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor, binding: CacheBinding,
+                    position: PositionEncoding) -> None:
+        if binding.kind != "state":
+            raise ValueError("a state-space mixer needs a state pool")
+        plain_residual(ctx, h, x)
+        n, ws = ctx.n_rows, ctx.workspace
+        n_req = ctx.cu_q.numel() - 1
+        pool = ctx.state_pools[binding.index]
+        u = ws.get("state_space_in", n, self.in_rows, ctx.dtype)
+        linear(ctx, h, self.in_weight, None, u, n)
+        xbc = ws.get("state_space_conv", n, self.conv_width, ctx.dtype)
+        kernels.short_conv(u, self.inner, self.conv_weight, self.conv_bias, pool[:, self.state_numel:], ctx.state_slots,
+                           ctx.cu_q, ctx.q_req, ctx.positions, n_req, xbc, 0, n, activation="silu")
+        sums = ws.get("state_space_sums", n, self.inner, torch.float32)
+        gn = self.n_group * self.state_dim
+        kernels.gated_state(xbc, self.inner + gn, self.inner, 0, self.n_head, self.n_group, self.state_dim, self.value_dim,
+                            u, self.dt_off, "head_softplus", pool[:, :self.state_numel], ctx.state_slots, ctx.cu_q, n_req,
+                            ctx.positions, sums, dt_bias=self.dt_bias, a_log=self.a_log, skip=self.skip)
+        y = ws.get("state_space_out", n, self.inner, ctx.dtype)
+        kernels.rms_norm(sums, self.norm_weight, y, n, self.norm_eps, self.inner // self.norm_groups,
+                         groups=self.norm_groups, gate=u, gate_act="silu_first")
         linear_add(ctx, y, self.out_weight, None, x, n)

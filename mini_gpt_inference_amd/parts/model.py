@@ -283,6 +283,7 @@ class DecoderModel:
                 if isinstance(need, KVNeed):
                     kv_runs.append(KVRun(int(getattr(part, "n_head", need.n_kv_head)), need.n_kv_head,
                                          need.head_dim, need.window, 1 if need.joint else 2))
+                    state_floats += int(need.state_numel)
                 elif isinstance(need, StateNeed):
                     state_floats += int(need.numel)
         return ModelCost(sum(size(name) for name in whole), row_bytes, run_elements, matrices(self.head),
@@ -332,7 +333,11 @@ class DecoderModel:
                         keys.append(key)
                         groups.append(CacheGroupSpec(key[0], key[1], key[2], 0, key[3]))
                     g = keys.index(key)
-                    bindings[role] = CacheBinding("kv", g, groups[g].n_pools, writes=True)
+                    state = -1
+                    if need.state_numel:
+                        state = len(state_numels)
+                        state_numels.append(int(need.state_numel))
+                    bindings[role] = CacheBinding("kv", g, groups[g].n_pools, writes=True, state=state)
                     groups[g] = CacheGroupSpec(key[0], key[1], key[2], groups[g].n_pools + 1, key[3])
                 elif isinstance(need, StateNeed):
                     bindings[role] = CacheBinding("state", -1, len(state_numels), writes=True)

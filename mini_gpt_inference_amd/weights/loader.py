@@ -68,7 +68,7 @@ def load_tensors(model_dir: str, wanted: Mapping[str, WeightRequest], compute_dt
         for name, req in wanted.items():
             if name in by_name:
                 shape = tuple(fh.get_slice(by_name[name]).get_shape())
-                if shape != tuple(req.shape):
+                if not req.fits(shape):
                     wrong.append((name, tuple(req.shape), shape))
         if missing or unexpected or wrong:
             lines = [f"{path} does not match the model that config.json describes:"]
