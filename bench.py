@@ -320,13 +320,39 @@ def bobevik_like(layers, width, heads, vocab):
             "layers": out}
 
 
-COMPARED = {"viperax": viperax_like, "bobevik": bobevik_like}
+def rilavik_like(layers, width, heads, vocab):
+    """A Rilavik config.json of a GPT-2-style model's size: the same layers, width and vocabulary, heads of
+    128 channels; parallel and gla layers in turn; every token goes through 8 width^2 feed-forward elements
+    a layer (2 of 8 experts of hidden size 4/3 width).  A parallel layer gives half the heads to a windowed
+    attention with a quarter as many key/value heads and short convolutions, half to the state-space mixer
+    (a state of 128 values a channel, two groups)."""
+    ff = width * 4 // 3 // 64 * 64
+    half = max(heads // 2, 1)
+    out = []
+    for i in range(layers):
+        if i % 2:
+            kind, mixer = "gla", {"heads": heads, "dim": 128, "vdim": 128, "tau": 16.0}
+        else:
+            kind = "parallel"
+            mixer = {"left": {"heads": half, "kv_heads": max(half // 4, 1), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                              "conv": 4, "mask": {"size": 512}, "rot": {"dims": 64, "base": 50000.0, "scaling": {"factor": 4.0}}},
+                     "right": {"heads": half, "vdim": 128, "state": 128, "groups": min(2, half), "conv": 4, "norm_groups": 1},
+                     "left_scale": 1.0, "right_scale": 1.0}
+        out.append({"type": kind, "mixer": mixer,
+                    "mlp": {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": ff}}})
+    return {"architecture": "Rilavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": out}
+
+
+COMPARED = {"viperax": viperax_like, "bobevik": bobevik_like, "rilavik": rilavik_like}
+# the model a design is measured beside: the GPT-2-style model, or the design nearest to it
+BESIDE = {"rilavik": "bobevik"}
 
 
 def compare_run(args, name):
-    """--compare viperax | bobevik: prefill (2 prompts of 1,024 tokens as one step) and decode (batch 8,
-    by the default run's timing rule, fewer blocks) of that design beside the GPT-2-style model at equal
-    layers, width, heads and vocabulary, random weights, at COMPARE_SIZES.  One JSON line."""
+    """--compare viperax | bobevik | rilavik: prefill (2 prompts of 1,024 tokens as one step) and decode
+    (batch 8, by the default run's timing rule, fewer blocks) of that design beside the GPT-2-style model
+    (Rilavik: beside Bobevik, the nearest design) at equal layers, width, heads and vocabulary, random
+    weights, at COMPARE_SIZES.  One JSON line."""
     import argparse as _argparse
     import gc
 
@@ -335,10 +361,13 @@ def compare_run(args, name):
     vocab, rows = 32768, []
     for layers, width, heads in COMPARE_SIZES:
         row = {"layers": layers, "width": width, "heads": heads, "vocab": vocab}
-        for label, raw in (("gpt2-mini", {"architecture": "gpt2-mini", "n_layer": layers, "n_embd": width,
-                                          "n_head": heads, "vocab_size": vocab, "block_size": args.positions,
-                                          "bias": True, "layer_norm_eps": 1e-5}),
-                           (name, COMPARED[name](layers, width, heads, vocab))):
+        beside = BESIDE.get(name, "gpt2-mini")
+        if beside == "gpt2-mini":
+            beside_raw = {"architecture": "gpt2-mini", "n_layer": layers, "n_embd": width, "n_head": heads,
+                          "vocab_size": vocab, "block_size": args.positions, "bias": True, "layer_norm_eps": 1e-5}
+        else:
+            beside_raw = COMPARED[beside](layers, width, heads, vocab)
+        for label, raw in ((beside, beside_raw), (name, COMPARED[name](layers, width, heads, vocab))):
             a = _argparse.Namespace(**vars(args))
             a.raw_config = raw
             pre = prefill_run(a, args.dtype, reps=10, warmups=5)
@@ -358,7 +387,8 @@ def compare_run(args, name):
             torch.cuda.empty_cache()
         rows.append(row)
         print(f"[bench] compared {row}", file=sys.stderr, flush=True)
-    return {"compare": f"{name} beside gpt2-mini at equal layers, width, heads and vocabulary", "dtype": args.dtype,
+    return {"compare": f"{name} beside {BESIDE.get(name, 'gpt2-mini')} at equal layers, width, heads and vocabulary",
+            "dtype": args.dtype,
             "batch": args.batch, "prompt_len": args.prompt, "prefill": "2 x 1024 tokens, one step", "rows": rows}
 
 

@@ -33,11 +33,12 @@ def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std_s
             order = torch.rand((shape[0], int(scale)), generator=gen).argsort(dim=1)
             tensors[name] = order[:, :shape[1]].to(torch.int32).contiguous()
             continue
+        if rule == "around":            # values near `scale`, whatever its sign
+            tensors[name] = (torch.empty(shape, dtype=torch.float32).normal_(0.0, 0.25, generator=gen) + scale).to(dtype)
+            continue
         t = torch.empty(shape, dtype=torch.float32).normal_(0.0, scale * std_scale, generator=gen)
         if rule == "gain":
             t += 1.0
-        elif rule == "around":          # values near `scale`
-            t = t * 0.25 + scale
         elif rule == "identity":        # a square matrix near the identity
             t += torch.eye(shape[0])
         elif rule != "normal":
