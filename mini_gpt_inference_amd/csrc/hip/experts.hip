@@ -139,9 +139,21 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const void* __restrict
   if (q_req && q_req[n] < 0) return;     // padded token
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   for (int e = wave; e < n_experts; e += 4) {
+    // eight columns a lane in flight at once (the sum takes them in rising order all the same)
     float acc = 0.f;
-    for (int c = lane; c < width; c += 64)
-      acc = fmaf(load_f(w, w_dtype, (long)e * width + c), load_f(h, dtype, (long)n * ldh + c), acc);
+    for (int c0 = lane; c0 < width; c0 += 64 * 8) {
+      float wv[8], hv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int c = c0 + 64 * u;
+        const bool ok = c < width;
+        wv[u] = ok ? load_f(w, w_dtype, (long)e * width + c) : 0.f;
+        hv[u] = ok ? load_f(h, dtype, (long)n * ldh + c) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (c0 + 64 * u < width) acc = fmaf(wv[u], hv[u], acc);
+    }
     acc = wave_sum(acc);
     if (lane == 0) logit[e] = acc;
   }

@@ -163,6 +163,11 @@ int mgpt_gated_state(const void* z, int dtype, long ldz, int q_off, int k_off, i
     int head_dim, int value_dim, const void* a, int a_dtype, long lda, int a_off, int mode, float q_scale, float inv_tau,
     const float* dt_bias, const float* a_log, const float* skip, float* state, long ld_state, const int* state_slots,
     const int* cu_q, int n_req, const int* positions, float* out, long ldo, hipStream_t stream);
+int mgpt_gated_state_chunked(const void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head, int n_group,
+                             int head_dim, int value_dim, const void* a, int a_dtype, long lda, int a_off, int mode,
+                             float q_scale, float inv_tau, const float* dt_bias, const float* a_log, const float* skip,
+                             float* state, long ld_state, const int* state_slots, const int* cu_q, int n_req, int n_tokens,
+                             const int* positions, float* qkg, float* out, long ldo, hipStream_t stream);
 // short_conv.hip
 int mgpt_short_conv(const void* u, int dtype, long ldu, int u_off, const float* w, const float* bias, int act,
     float* state, long ld_state, const int* state_slots, const int* cu_q, const int* q_req, const int* positions,
@@ -236,4 +241,5 @@ int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_st
   X(mgpt_router_topk) \
   X(mgpt_gather_scale_rows) \
   X(mgpt_gated_state) \
+  X(mgpt_gated_state_chunked) \
   X(mgpt_short_conv)

@@ -64,14 +64,14 @@ __global__ __launch_bounds__(256) void short_conv_state_kernel(
 }
 
 // u: rows in `dtype`, the C channels at u_off; w: float32 [C][J]; bias: float32 [C] or null; act: 0 none, 1 silu.
-// state: rows of ld_state floats, (J - 1) * C of them used.  out: rows in out_dtype, the C channels at o_off
+// state: rows of ld_state floats, (J - 1) * C of them used (with one tap none: it may be null).  out: rows in out_dtype, the C channels at o_off
 // (not the rows of u: a token reads the inputs of the tokens before it).
 extern "C" int mgpt_short_conv(const void* u, int dtype, long ldu, int u_off, const float* w, const float* bias, int act,
                                float* state, long ld_state, const int* state_slots, const int* cu_q, const int* q_req,
                                const int* positions, int n_req, void* out, int out_dtype, long ldo, int o_off,
                                int n_tokens, int channels, int taps, hipStream_t stream) {
   if (n_tokens == 0 || n_req == 0) return MGPT_OK;
-  if (!u || !w || !state || !state_slots || !cu_q || !q_req || !positions || !out) return MGPT_ERR_NULL;
+  if (!u || !w || (!state && taps > 1) || !state_slots || !cu_q || !q_req || !positions || !out) return MGPT_ERR_NULL;
   if (!dtype_ok(dtype) || !dtype_ok(out_dtype)) return MGPT_ERR_BAD_DTYPE;
   if (n_tokens < 0 || n_req < 0 || channels <= 0 || taps < 1 || taps > SC_MAX_TAPS || (act != 0 && act != 1) ||
       ld_state < (long)(taps - 1) * channels || u == out)

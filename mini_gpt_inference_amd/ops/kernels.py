@@ -1536,6 +1536,48 @@ def gated_state(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int
     _check(rc, "gated_state")
 
 
+def gated_state_chunked(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int, n_group: int, head_dim: int,
+                        value_dim: int, a: torch.Tensor, a_off: int, mode: str, state: torch.Tensor,
+                        state_slots: torch.Tensor, cu_q: torch.Tensor, n_req: int, n_tokens: int, positions: torch.Tensor,
+                        qkg: torch.Tensor, out: torch.Tensor, q_scale: float = 1.0, tau: float = 1.0,
+                        dt_bias: Optional[torch.Tensor] = None, a_log: Optional[torch.Tensor] = None,
+                        skip: Optional[torch.Tensor] = None) -> bool:
+    """gated_state for steps with prompt portions: the recurrence 32 tokens at a time as float32 matrix products,
+    the decays between a chunk's tokens from sums of their logarithms.  qkg: float32 scratch [>= n_tokens,
+    3 * heads * dim].  False, with nothing launched, for head sizes beyond CHUNKED_STATE_MAX_DIM."""
+    if head_dim > CHUNKED_STATE_MAX_DIM:
+        return False
+    _need_cuda(z, a, state, state_slots, cu_q, positions, out, qkg, dt_bias, a_log, skip)
+    _need(mode in GATED_STATE_MODES, f"gated_state: mode {mode!r} is none of {sorted(GATED_STATE_MODES)}")
+    _rows_2d("gated_state z", z, n_tokens)
+    _rows_2d("gated_state a", a, n_tokens)
+    _need(n_head % n_group == 0, "gated_state: heads must be a multiple of groups")
+    _need(z.shape[1] >= max(q_off, k_off) + n_group * head_dim and z.shape[1] >= v_off + n_head * value_dim,
+          "gated_state: z is too narrow")
+    _need(a.shape[1] >= a_off + (n_head * head_dim if mode == "channel_sigmoid" else n_head), "gated_state: a is too narrow")
+    _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] >= n_tokens
+          and out.shape[1] >= n_head * value_dim, "gated_state: out must be float32 rows of all heads' values")
+    _need(qkg.dtype == torch.float32 and qkg.is_contiguous() and qkg.dim() == 2 and qkg.shape[0] >= n_tokens
+          and qkg.shape[1] == 3 * n_head * head_dim, "gated_state_chunked: qkg must be float32 [tokens, 3 * heads * dim]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] == n_head * head_dim * value_dim, "gated_state: state must be float32 rows of heads * dim * vdim")
+    for name, t in (("dt_bias", dt_bias), ("a_log", a_log), ("skip", skip)):
+        _need(t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n_head),
+              f"gated_state: {name} must be float32 [heads]")
+    _need(mode != "head_softplus" or (dt_bias is not None and a_log is not None), "gated_state: this mode needs dt_bias and a_log")
+    _need(0 < value_dim <= 256 and tau > 0.0, "gated_state takes value sizes up to 256")
+    _need_i32("state_slots", state_slots, n_req)
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need_i32("positions", positions, n_tokens)
+    rc = library.kernels().mgpt_gated_state_chunked(
+        _ptr(z), _dtype_code(z), z.stride(0), q_off, k_off, v_off, n_head, n_group, head_dim, value_dim, _ptr(a),
+        _dtype_code(a), a.stride(0), a_off, GATED_STATE_MODES[mode], float(q_scale), 1.0 / float(tau), _ptr(dt_bias),
+        _ptr(a_log), _ptr(skip), _ptr(state), state.stride(0), _ptr(state_slots), _ptr(cu_q), n_req, n_tokens,
+        _ptr(positions), _ptr(qkg), _ptr(out), out.stride(0), _stream())
+    _check(rc, "gated_state_chunked", 2)
+    return True
+
+
 MAX_CONV_TAPS = 9
 CONV_ACTIVATIONS = {None: 0, "silu": 1}
 

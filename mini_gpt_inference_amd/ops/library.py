@@ -175,6 +175,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_gather_scale_rows": [P, I, L, P, P, P, P, L, I, I, P],
         # a state with a decay made from the token, short convolutions
         "mgpt_gated_state": [P, I, L, I, I, I, I, I, I, I, P, I, L, I, I, F, F, P, P, P, P, L, P, P, I, P, P, L, P],
+        "mgpt_gated_state_chunked": [P, I, L, I, I, I, I, I, I, I, P, I, L, I, I, F, F, P, P, P, P, L, P, P, I, I, P, P, P, L, P],
         "mgpt_short_conv": [P, I, L, I, P, P, I, P, L, P, P, P, P, I, P, I, L, I, I, I, I, P],
     }
     for name, argtypes in table.items():

@@ -590,9 +590,19 @@ class GatedLinearAttention(Mixer):
         u = ws.get("gla_decay", n, self.qk_width, ctx.dtype)
         linear(ctx, z[:, self.a_off:], self.decay_out_weight, self.decay_out_bias, u, n)
         sums = ws.get("gla_sums", n, self.v_width, torch.float32)
-        kernels.gated_state(z, 0, self.k_off, self.v_off, self.n_head, self.n_head, self.head_dim, self.value_dim, u, 0,
-                            "channel_sigmoid", ctx.state_pools[binding.index], ctx.state_slots, ctx.cu_q,
-                            ctx.cu_q.numel() - 1, ctx.positions, sums, q_scale=self.q_scale, tau=self.tau)
+        state, n_req = ctx.state_pools[binding.index], ctx.cu_q.numel() - 1
+        # a step with prompt portions: the recurrence a chunk of tokens at a time on the matrix cores; single
+        # tokens: token by token
+        chunked = False
+        if not ctx.decode_only and self.head_dim <= kernels.CHUNKED_STATE_MAX_DIM:
+            qkg = ws.get("gated_state_qkg", n, 3 * self.qk_width, torch.float32)
+            chunked = kernels.gated_state_chunked(z, 0, self.k_off, self.v_off, self.n_head, self.n_head, self.head_dim,
+                                                  self.value_dim, u, 0, "channel_sigmoid", state, ctx.state_slots, ctx.cu_q,
+                                                  n_req, n, ctx.positions, qkg, sums, q_scale=self.q_scale, tau=self.tau)
+        if not chunked:
+            kernels.gated_state(z, 0, self.k_off, self.v_off, self.n_head, self.n_head, self.head_dim, self.value_dim, u, 0,
+                                "channel_sigmoid", state, ctx.state_slots, ctx.cu_q, n_req, ctx.positions, sums,
+                                q_scale=self.q_scale, tau=self.tau)
         y = ws.get("gla_out", n, self.v_width, ctx.dtype)
         kernels.rms_norm(sums, self.head_gain, y, n, self.norm_eps, self.value_dim, groups=self.n_head,
                          gate=z[:, self.g_off:], gate_act="silu")
@@ -661,9 +671,18 @@ class StateSpaceMixer(Mixer):
                            ctx.cu_q, ctx.q_req, ctx.positions, n_req, xbc, 0, n, activation="silu")
         sums = ws.get("state_space_sums", n, self.inner, torch.float32)
         gn = self.n_group * self.state_dim
-        kernels.gated_state(xbc, self.inner + gn, self.inner, 0, self.n_head, self.n_group, self.state_dim, self.value_dim,
-                            u, self.dt_off, "head_softplus", pool[:, :self.state_numel], ctx.state_slots, ctx.cu_q, n_req,
-                            ctx.positions, sums, dt_bias=self.dt_bias, a_log=self.a_log, skip=self.skip)
+        state = pool[:, :self.state_numel]
+        chunked = False
+        if not ctx.decode_only and self.state_dim <= kernels.CHUNKED_STATE_MAX_DIM:
+            qkg = ws.get("gated_state_qkg", n, 3 * self.n_head * self.state_dim, torch.float32)
+            chunked = kernels.gated_state_chunked(xbc, self.inner + gn, self.inner, 0, self.n_head, self.n_group,
+                                                  self.state_dim, self.value_dim, u, self.dt_off, "head_softplus", state,
+                                                  ctx.state_slots, ctx.cu_q, n_req, n, ctx.positions, qkg, sums,
+                                                  dt_bias=self.dt_bias, a_log=self.a_log, skip=self.skip)
+        if not chunked:
+            kernels.gated_state(xbc, self.inner + gn, self.inner, 0, self.n_head, self.n_group, self.state_dim,
+                                self.value_dim, u, self.dt_off, "head_softplus", state, ctx.state_slots, ctx.cu_q, n_req,
+                                ctx.positions, sums, dt_bias=self.dt_bias, a_log=self.a_log, skip=self.skip)
         y = ws.get("state_space_out", n, self.inner, ctx.dtype)
         kernels.rms_norm(sums, self.norm_weight, y, n, self.norm_eps, self.inner // self.norm_groups,
                          groups=self.norm_groups, gate=u, gate_act="silu_first")

@@ -199,11 +199,22 @@ def right_mixer(h: torch.Tensor, tensors: Dict[str, torch.Tensor], p: str, m: di
 
 
 # ---------------------------------------------------------------- feed-forward
+# With ROUTER_GAPS a list, every call of routed_experts appends one number per token: by how much the router's
+# choice is decided.  A test that compares with reduced precision leaves out the tokens whose choice hangs on
+# less than that precision can tell.
+ROUTER_GAPS: Optional[list] = None
+
+
 def routed_experts(h: torch.Tensor, tensors: Dict[str, torch.Tensor], p: str, mlp: dict) -> torch.Tensor:
     """Scores s = sigmoid(router h); a token's `top` experts are those with the largest scores; the output is
     the sum over them of expert(s_e h), expert(u) = down (silu(gate u) * (up u))."""
     n, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
-    scores = sigmoid(_r(h) @ tensors[p + "router"].T)
+    logits = _r(h) @ tensors[p + "router"].T
+    if ROUTER_GAPS is not None:
+        # how decided each token's choice is: the last chosen logit minus the first one left out
+        srt = torch.sort(logits, dim=-1, descending=True).values
+        ROUTER_GAPS.append(srt[:, top - 1] - srt[:, top] if top < n else torch.full((h.shape[0],), math.inf, dtype=DTYPE))
+    scores = sigmoid(logits)
     chosen = torch.topk(scores, top, dim=-1).indices
     out = torch.zeros_like(h)
     for e in range(n):
