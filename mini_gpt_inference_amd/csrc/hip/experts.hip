@@ -130,10 +130,14 @@ extern "C" int mgpt_gather_rows(const void* src, long ld, const int* slot_token,
 // chosen[n][c] is the expert with the c-th largest score (of equal scores the lower number first) and
 // weight[n][c] its score.  One workgroup a token: a wave an expert at a time, lanes along the width in a
 // fixed order, then the first wave picks the largest `top` times.
-__global__ __launch_bounds__(256) void router_topk_kernel(const void* __restrict__ h, int dtype, long ldh,
-                                                          const void* __restrict__ w, int w_dtype, const int* __restrict__ q_req,
-                                                          int width, int n_experts, int top, int kind,
-                                                          int* __restrict__ chosen, float* __restrict__ weight) {
+__device__ __forceinline__ float router_value(float v) { return v; }
+__device__ __forceinline__ float router_value(bf16_t v) { return bf16_to_float(v); }
+
+// (the storage types are the kernel's parameters: a choice made load by load keeps the loads from being in flight together)
+template <typename HT, typename WT>
+__global__ __launch_bounds__(256) void router_topk_kernel(const HT* __restrict__ h, long ldh, const WT* __restrict__ w,
+                                                          const int* __restrict__ q_req, int width, int n_experts, int top,
+                                                          int kind, int* __restrict__ chosen, float* __restrict__ weight) {
   __shared__ float logit[EX_MAX_EXPERTS];
   const int n = blockIdx.x;
   if (q_req && q_req[n] < 0) return;     // padded token
@@ -147,8 +151,8 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const void* __restrict
       for (int u = 0; u < 8; ++u) {
         const int c = c0 + 64 * u;
         const bool ok = c < width;
-        wv[u] = ok ? load_f(w, w_dtype, (long)e * width + c) : 0.f;
-        hv[u] = ok ? load_f(h, dtype, (long)n * ldh + c) : 0.f;
+        wv[u] = ok ? router_value(w[(long)e * width + c]) : 0.f;
+        hv[u] = ok ? router_value(h[(long)n * ldh + c]) : 0.f;
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u)
@@ -193,8 +197,14 @@ extern "C" int mgpt_router_topk(const void* h, int dtype, long ldh, const void* 
   if (n_rows < 0 || width <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || top <= 0 || top > n_experts ||
       (kind != 0 && kind != 1))
     return MGPT_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(router_topk_kernel, dim3(n_rows), dim3(256), 0, stream, h, dtype, ldh, w, w_dtype, q_req, width,
-                     n_experts, top, kind, chosen, weight);
+#define ROUTER_LAUNCH(HT, WT)                                                                                        \
+  hipLaunchKernelGGL((router_topk_kernel<HT, WT>), dim3(n_rows), dim3(256), 0, stream, (const HT*)h, ldh, (const WT*)w, \
+                     q_req, width, n_experts, top, kind, chosen, weight)
+  if (dtype == MGPT_F32 && w_dtype == MGPT_F32) ROUTER_LAUNCH(float, float);
+  else if (dtype == MGPT_F32) ROUTER_LAUNCH(float, bf16_t);
+  else if (w_dtype == MGPT_F32) ROUTER_LAUNCH(bf16_t, float);
+  else ROUTER_LAUNCH(bf16_t, bf16_t);
+#undef ROUTER_LAUNCH
   return mgpt_last_error();
 }
 
