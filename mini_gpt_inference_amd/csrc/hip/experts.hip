@@ -128,40 +128,73 @@ extern "C" int mgpt_gather_rows(const void* src, long ld, const int* slot_token,
 // A router: scores of every expert for a token, in float32 whatever the rows' dtype, and the `top`
 // largest.  logit[e] = w[e] . h; score = sigmoid(logit) (kind 0) or the logit itself (kind 1);
 // chosen[n][c] is the expert with the c-th largest score (of equal scores the lower number first) and
-// weight[n][c] its score.  One workgroup a token: a wave an expert at a time, lanes along the width in a
-// fixed order, then the first wave picks the largest `top` times.
+// weight[n][c] its score.  One workgroup a token: its threads along the width in a fixed order, then the first
+// wave picks the largest `top` times.
 __device__ __forceinline__ float router_value(float v) { return v; }
 __device__ __forceinline__ float router_value(bf16_t v) { return bf16_to_float(v); }
 
-// (the storage types are the kernel's parameters: a choice made load by load keeps the loads from being in flight together)
-template <typename HT, typename WT>
+__device__ __forceinline__ void router_load8(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void router_load8(const bf16_t* p, float (&v)[8]) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  const unsigned words[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    v[2 * k] = __uint_as_float(words[k] << 16);
+    v[2 * k + 1] = __uint_as_float(words[k] & 0xffff0000u);
+  }
+}
+
+// The storage types are the kernel's parameters (a choice made load by load keeps the loads from being in flight
+// together).  VEC: the width is a multiple of 8 and the rows are aligned for loads of eight elements; then thread t
+// takes columns 8 t .. 8 t + 7 of every stretch of 2,048 columns for eight experts at a time, whose loads are all in
+// flight together, and the sums meet through the waves in a fixed order.  Otherwise a wave takes an expert at a time.
+template <typename HT, typename WT, bool VEC>
 __global__ __launch_bounds__(256) void router_topk_kernel(const HT* __restrict__ h, long ldh, const WT* __restrict__ w,
                                                           const int* __restrict__ q_req, int width, int n_experts, int top,
                                                           int kind, int* __restrict__ chosen, float* __restrict__ weight) {
   __shared__ float logit[EX_MAX_EXPERTS];
+  __shared__ float part[4][8];
   const int n = blockIdx.x;
   if (q_req && q_req[n] < 0) return;     // padded token
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int e = wave; e < n_experts; e += 4) {
-    // eight columns a lane in flight at once (the sum takes them in rising order all the same)
-    float acc = 0.f;
-    for (int c0 = lane; c0 < width; c0 += 64 * 8) {
-      float wv[8], hv[8];
+  if (VEC) {
+    for (int e0 = 0; e0 < n_experts; e0 += 8) {
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int c = 8 * threadIdx.x; c < width; c += 8 * 256) {
+        float hv[8];
+        router_load8(h + (long)n * ldh + c, hv);
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int c = c0 + 64 * u;
-        const bool ok = c < width;
-        wv[u] = ok ? router_value(w[(long)e * width + c]) : 0.f;
-        hv[u] = ok ? router_value(h[(long)n * ldh + c]) : 0.f;
+        for (int j = 0; j < 8; ++j) {
+          const int e = e0 + j < n_experts ? e0 + j : n_experts - 1;     // (behind the last expert: loaded again, not used)
+          float wv[8];
+          router_load8(w + (long)e * width + c, wv);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc[j] = fmaf(wv[k], hv[k], acc[j]);
+        }
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (c0 + 64 * u < width) acc = fmaf(wv[u], hv[u], acc);
+      for (int j = 0; j < 8; ++j) {
+        const float sum = wave_sum(acc[j]);
+        if (lane == 0) part[wave][j] = sum;
+      }
+      __syncthreads();
+      if (threadIdx.x < 8 && e0 + threadIdx.x < n_experts)
+        logit[e0 + threadIdx.x] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+      __syncthreads();
     }
-    acc = wave_sum(acc);
-    if (lane == 0) logit[e] = acc;
+  } else {
+    for (int e = wave; e < n_experts; e += 4) {
+      float acc = 0.f;
+      for (int c = lane; c < width; c += 64)
+        acc = fmaf(router_value(w[(long)e * width + c]), router_value(h[(long)n * ldh + c]), acc);
+      acc = wave_sum(acc);
+      if (lane == 0) logit[e] = acc;
+    }
+    __syncthreads();
   }
-  __syncthreads();
   if (wave != 0) return;
   for (int c = 0; c < top; ++c) {
     float best = -INFINITY;
@@ -197,13 +230,21 @@ extern "C" int mgpt_router_topk(const void* h, int dtype, long ldh, const void* 
   if (n_rows < 0 || width <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || top <= 0 || top > n_experts ||
       (kind != 0 && kind != 1))
     return MGPT_ERR_BAD_SHAPE;
-#define ROUTER_LAUNCH(HT, WT)                                                                                        \
-  hipLaunchKernelGGL((router_topk_kernel<HT, WT>), dim3(n_rows), dim3(256), 0, stream, (const HT*)h, ldh, (const WT*)w, \
-                     q_req, width, n_experts, top, kind, chosen, weight)
-  if (dtype == MGPT_F32 && w_dtype == MGPT_F32) ROUTER_LAUNCH(float, float);
-  else if (dtype == MGPT_F32) ROUTER_LAUNCH(float, bf16_t);
-  else if (w_dtype == MGPT_F32) ROUTER_LAUNCH(bf16_t, float);
-  else ROUTER_LAUNCH(bf16_t, bf16_t);
+  const size_t h_size = dtype == MGPT_F32 ? 4 : 2, w_size = w_dtype == MGPT_F32 ? 4 : 2;
+  const bool vec = !(width & 7) && !(((size_t)h | (size_t)(ldh * h_size)) & 15) && !((size_t)w & 15);
+#define ROUTER_LAUNCH(HT, WT)                                                                                            \
+  {                                                                                                                      \
+    if (vec)                                                                                                             \
+      hipLaunchKernelGGL((router_topk_kernel<HT, WT, true>), dim3(n_rows), dim3(256), 0, stream, (const HT*)h, ldh,      \
+                         (const WT*)w, q_req, width, n_experts, top, kind, chosen, weight);                              \
+    else                                                                                                                 \
+      hipLaunchKernelGGL((router_topk_kernel<HT, WT, false>), dim3(n_rows), dim3(256), 0, stream, (const HT*)h, ldh,     \
+                         (const WT*)w, q_req, width, n_experts, top, kind, chosen, weight);                              \
+  }
+  if (dtype == MGPT_F32 && w_dtype == MGPT_F32) ROUTER_LAUNCH(float, float)
+  else if (dtype == MGPT_F32) ROUTER_LAUNCH(float, bf16_t)
+  else if (w_dtype == MGPT_F32) ROUTER_LAUNCH(bf16_t, float)
+  else ROUTER_LAUNCH(bf16_t, bf16_t)
 #undef ROUTER_LAUNCH
   return mgpt_last_error();
 }
@@ -222,6 +263,27 @@ __global__ void gather_scale_rows_kernel(const void* __restrict__ src, int dtype
   store_f(sorted, dtype, s * lds + c, pair_weight[slot_pair[s]] * load_f(src, dtype, (long)row * ld + c));
 }
 
+// the same for bfloat16 rows of a multiple of 8 elements, 16-byte aligned: eight elements a lane
+__global__ void gather_scale_rows_bf16x8_kernel(const uint4* __restrict__ src, long ld16, const int* __restrict__ slot_token,
+                                                const int* __restrict__ slot_pair, const float* __restrict__ pair_weight,
+                                                uint4* __restrict__ sorted, long lds16, int n_slots, int chunks) {
+  const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (i >= (long)n_slots * chunks) return;
+  const long s = i / chunks;
+  const int c = (int)(i - s * chunks);
+  const int row = slot_token[s];
+  if (row < 0) return;
+  const float wgt = pair_weight[slot_pair[s]];
+  uint4 v = src[row * ld16 + c];
+  unsigned* words = reinterpret_cast<unsigned*>(&v);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float lo = __uint_as_float(words[k] << 16) * wgt, hi = __uint_as_float(words[k] & 0xffff0000u) * wgt;
+    words[k] = (unsigned)float_to_bf16(lo) | ((unsigned)float_to_bf16(hi) << 16);
+  }
+  sorted[s * lds16 + c] = v;
+}
+
 extern "C" int mgpt_gather_scale_rows(const void* src, int dtype, long ld, const int* slot_token, const int* slot_pair,
                                       const float* pair_weight, void* sorted, long lds, int n_slots, int width,
                                       hipStream_t stream) {
@@ -229,6 +291,13 @@ extern "C" int mgpt_gather_scale_rows(const void* src, int dtype, long ld, const
   if (!src || !slot_token || !slot_pair || !pair_weight || !sorted) return MGPT_ERR_NULL;
   if (!dtype_ok(dtype)) return MGPT_ERR_BAD_DTYPE;
   if (n_slots < 0 || width <= 0 || ld < width || lds < width) return MGPT_ERR_BAD_SHAPE;
+  if (dtype == MGPT_BF16 && !(width & 7) && !(ld & 7) && !(lds & 7) && !(((size_t)src | (size_t)sorted) & 15)) {
+    const long blocks8 = ((long)n_slots * (width / 8) + 255) / 256;
+    if (blocks8 > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(gather_scale_rows_bf16x8_kernel, dim3((unsigned)blocks8), dim3(256), 0, stream, (const uint4*)src,
+                       ld / 8, slot_token, slot_pair, pair_weight, (uint4*)sorted, lds / 8, n_slots, width / 8);
+    return mgpt_last_error();
+  }
   const long total = (long)n_slots * width;
   const long blocks = (total + 255) / 256;
   if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;

@@ -14,11 +14,13 @@
 
 #define SC_MAX_TAPS 9
 
+// (the storage types are the kernel's parameters, so that a thread's loads of all taps are in flight together)
+template <typename UT, typename OT>
 __global__ __launch_bounds__(256) void short_conv_kernel(
-    const void* __restrict__ u, int dtype, long ldu, int u_off, const float* __restrict__ w, const float* __restrict__ bias,
+    const UT* __restrict__ u, long ldu, int u_off, const float* __restrict__ w, const float* __restrict__ bias,
     int act, const float* __restrict__ state, long ld_state, const int* __restrict__ state_slots,
-    const int* __restrict__ cu_q, const int* __restrict__ q_req, const int* __restrict__ positions, void* __restrict__ out,
-    int out_dtype, long ldo, int o_off, int C, int J) {
+    const int* __restrict__ cu_q, const int* __restrict__ q_req, const int* __restrict__ positions, OT* __restrict__ out,
+    long ldo, int o_off, int C, int J) {
   const int n = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   const int r = q_req[n];
@@ -30,13 +32,13 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
     if (p - back < 0) continue;     // before the sequence's start
     const int s = n - back;
     float val;
-    if (s >= start) val = load_f(u, dtype, (long)s * ldu + u_off + c);
+    if (s >= start) val = to_float<UT>(u[(long)s * ldu + u_off + c]);
     else if (slot >= 0) val = state[(long)slot * ld_state + (long)((J - 1) - (start - s)) * C + c];
     else val = 0.f;
     acc = fmaf(w[(long)c * J + j], val, acc);
   }
   if (act == 1) acc = acc / (1.0f + expf(-acc));
-  store_f(out, out_dtype, (long)n * ldo + o_off + c, acc);
+  out[(long)n * ldo + o_off + c] = from_float<OT>(acc);
 }
 
 // the request's last J - 1 inputs after this step: from the step's rows, or moved up inside the state
@@ -78,8 +80,14 @@ extern "C" int mgpt_short_conv(const void* u, int dtype, long ldu, int u_off, co
     return MGPT_ERR_BAD_SHAPE;
   const int cb = (channels + 255) / 256;
   if (cb > 65535) return MGPT_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(short_conv_kernel, dim3(n_tokens, cb), dim3(256), 0, stream, u, dtype, ldu, u_off, w, bias, act, state,
-                     ld_state, state_slots, cu_q, q_req, positions, out, out_dtype, ldo, o_off, channels, taps);
+#define SC_LAUNCH(UT, OT)                                                                                                 \
+  hipLaunchKernelGGL((short_conv_kernel<UT, OT>), dim3(n_tokens, cb), dim3(256), 0, stream, (const UT*)u, ldu, u_off, w, \
+                     bias, act, state, ld_state, state_slots, cu_q, q_req, positions, (OT*)out, ldo, o_off, channels, taps)
+  if (dtype == MGPT_F32 && out_dtype == MGPT_F32) SC_LAUNCH(float, float);
+  else if (dtype == MGPT_F32) SC_LAUNCH(float, bf16_t);
+  else if (out_dtype == MGPT_F32) SC_LAUNCH(bf16_t, float);
+  else SC_LAUNCH(bf16_t, bf16_t);
+#undef SC_LAUNCH
   if (taps > 1)
     hipLaunchKernelGGL(short_conv_state_kernel, dim3(n_req, cb), dim3(256), 0, stream, u, dtype, ldu, u_off, state, ld_state,
                        state_slots, cu_q, channels, taps);

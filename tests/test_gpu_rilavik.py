@@ -219,7 +219,8 @@ def test_the_state_far_back_matters(chunked):
 # ---------------------------------------------------------------- the router and the scaled rows
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("n,width,experts,top", [(1, 64, 2, 1), (9, 40, 5, 2), (70, 256, 12, 1), (33, 136, 9, 3),
-                                                 (5, 2048, 8, 2), (4, 24, 3, 3), (300, 96, 33, 4)])
+                                                 (5, 2048, 8, 2), (4, 24, 3, 3), (300, 96, 33, 4), (7, 100, 6, 2), (3, 4100, 9, 2),
+                                                 (2, 4096, 17, 3)])
 def test_router_picks_the_largest_scores(dtype, n, width, experts, top):
     g = torch.Generator().manual_seed(n + experts)
     h = _rnd(g, n + 1, width + 8, dtype=dtype)
