@@ -170,6 +170,7 @@ extern "C" int mgpt_gated_state(const void* z, int dtype, long ldz, int q_off, i
 #define GC_C 32        // tokens a chunk
 #define GC_DMAX 128    // largest head size of this path
 #define GC_LDP (GC_C + 4)
+#define GC_MILD 96.f   // a half chunk's decay, in powers of two, up to which 2^(L_start - L_j) is safely finite
 
 typedef float gs_f32x4 __attribute__((ext_vector_type(4)));
 
@@ -288,9 +289,10 @@ __global__ __launch_bounds__(256) void gated_state_chunk_kernel(
     fetch(t0 + GC_C);     // (behind the last chunk: no token is left, nothing is loaded)
     // ---- L: the logarithms summed over the chunk's tokens, each half by one thread per channel, then the first
     // half's total onto the second.  (Rows behind the chunk's last token hold zeros: L stays what it was there.)
+    int mild;
     {
       const int d = tid & 127, half = tid >> 7;
-      float run[16];
+      float run[16] = {};
       if (d < Dp) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) run[i] = Ls[(half * 16 + i) * ld + d];
@@ -301,7 +303,9 @@ __global__ __launch_bounds__(256) void gated_state_chunk_kernel(
           for (int i = 0; i < 16; ++i) Ls[i * ld + d] = run[i];
         }
       }
-      __syncthreads();
+      // do all channels keep at least 2^-GC_MILD of their size over each half?  Then the decay inside a half can be
+      // split at the half's start as well, without overflow on the key's side
+      mild = __syncthreads_and(SCALAR || d >= Dp || run[15] > -GC_MILD);
       if (d < Dp && half == 1) {
         const float first = Ls[15 * ld + d];
 #pragma unroll
@@ -335,6 +339,31 @@ __global__ __launch_bounds__(256) void gated_state_chunk_kernel(
         }
 #pragma unroll
         for (int v = 0; v < 4; ++v) Ps[(ti * 16 + 4 * g + v) * GC_LDP + tj * 16 + r16] = acc[v];
+      } else if (!SCALAR && mild) {
+        // a tile on the diagonal whose decays are mild: split at the start of the half (L = 0 before the chunk)
+        const float* lq = Ls + (ti * 16 + r16) * ld;
+        const float* lm = Ls + 15 * ld;
+#pragma unroll 2
+        for (int k0 = 0; k0 < Dp; k0 += 16) {
+          const int c = k0 + 4 * g;
+          gs_f32x4 a = *reinterpret_cast<const gs_f32x4*>(qrow + c), b = *reinterpret_cast<const gs_f32x4*>(krow + c);
+          const gs_f32x4 la = *reinterpret_cast<const gs_f32x4*>(lq + c);
+          gs_f32x4 mid = {0.f, 0.f, 0.f, 0.f};
+          if (ti) mid = *reinterpret_cast<const gs_f32x4*>(lm + c);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float w = gs_exp2(la[e] - mid[e]);     // (a tile on the diagonal: q's row and k's row are the same)
+            a[e] *= w;
+            b[e] *= __builtin_amdgcn_rcpf(w);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int i = ti * 16 + 4 * g + v, j = tj * 16 + r16;
+          Ps[i * GC_LDP + j] = j <= i ? acc[v] : 0.f;
+        }
       } else {
         // a tile on the diagonal: q . k without decay, which is what its diagonal needs; below it, with one decay a
         // head, the decay of the distance multiplies the sum; with a decay per channel the pairs' own threads fill in
@@ -359,7 +388,7 @@ __global__ __launch_bounds__(256) void gated_state_chunk_kernel(
 #pragma unroll
       for (int v = 0; v < 4; ++v) Ps[(ti * 16 + 4 * g + v) * GC_LDP + tj * 16 + r16] = 0.f;
     }
-    if (has_pair) {
+    if (has_pair && !mild) {
       const float* qrow = Qs + pi * ld;
       const float* krow = Ks + pj * ld;
       const float* lq = Ls + pi * ld;
