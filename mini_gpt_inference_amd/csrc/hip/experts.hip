@@ -432,20 +432,20 @@ extern "C" int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, c
   return mgpt_last_error();
 }
 
-// The grouped product in bfloat16 on the MFMA units, for tiles of 64 slots.  A workgroup owns a
-// tile x 64 (or 256) columns, a wave 16 (or 64) of the columns for all 64 slots: per 32 k one (or four)
-// slices of the expert's matrix (first operand) and four slices of gathered rows, 16 bytes a lane
-// straight from memory.
+// The grouped product in bfloat16 on the MFMA units, for tiles of 64 or 16 slots.  A workgroup owns a
+// tile x 64 (or 256) columns, a wave 16 (or 64) of the columns for all of the tile's slots: per 32 k one
+// (or four) slices of the expert's matrix (first operand) and four slices of gathered rows (one for a
+// tile of 16 slots: a decode step's few pairs an expert), 16 bytes a lane straight from memory.
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short ex_bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float ex_f32x4_t;
 
-template <typename OT, int NJ>
+template <typename OT, int NJ, int NT>     // NT: slices of 16 slots a tile
 __global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
     const bf16_t* __restrict__ A, long lda, const int* __restrict__ a_rows, const bf16_t* __restrict__ W,
     long w_stride, const int* __restrict__ tile_expert, const int* __restrict__ slot_token, OT* __restrict__ out,
     long ldo, const int* __restrict__ out_rows, int n_out, int k_dim) {
-  // a wave owns 64 slots x NJ * 16 columns: per 32 k it loads NJ slices of the matrix and four of the
-  // rows for 4 * NJ MFMAs
+  // a wave owns NT * 16 slots x NJ * 16 columns: per 32 k it loads NJ slices of the matrix and NT of the
+  // rows for NT * NJ MFMAs
   const int tile = blockIdx.y;
   const int e = tile_expert[tile];
   if (e < 0) return;
@@ -460,36 +460,36 @@ __global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
     w_ok[j] = col0 + j * 16 + li < n_out;
     wrow[j] = W + (long)e * w_stride + (long)(w_ok[j] ? col0 + j * 16 + li : 0) * k_dim;
   }
-  const bf16_t* arow[4];
-  bool a_ok[4];
-  long orow[4];
+  const bf16_t* arow[NT];
+  bool a_ok[NT];
+  long orow[NT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int slot = tile * 64 + 16 * t + li;
+  for (int t = 0; t < NT; ++t) {
+    const int slot = tile * (16 * NT) + 16 * t + li;
     a_ok[t] = slot_token[slot] >= 0;
     arow[t] = A + (a_ok[t] ? (long)(a_rows ? a_rows[slot] : slot) : 0L) * lda;
     orow[t] = a_ok[t] ? (long)(out_rows ? out_rows[slot] : slot) : 0L;
   }
   const ex_bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  ex_f32x4_t acc[NJ][4];
+  ex_f32x4_t acc[NJ][NT];
 #pragma unroll
   for (int j = 0; j < NJ; ++j)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[j][t] = ex_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NT; ++t) acc[j][t] = ex_f32x4_t{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < k_dim; k0 += 32) {
     const int k = k0 + lg * 8;
     const bool k_ok = k < k_dim;
-    ex_bf16x8_t wf[NJ], af[4];
+    ex_bf16x8_t wf[NJ], af[NT];
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
       wf[j] = (w_ok[j] && k_ok) ? *reinterpret_cast<const ex_bf16x8_t*>(wrow[j] + k) : zero;
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < NT; ++t)
       af[t] = (a_ok[t] && k_ok) ? *reinterpret_cast<const ex_bf16x8_t*>(arow[t] + k) : zero;
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < NT; ++t)
         acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[t], acc[j][t], 0, 0, 0);
   }
 #pragma unroll
@@ -497,7 +497,7 @@ __global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
     const int c = col0 + j * 16 + lg * 4;
     if (c >= n_out) continue;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < NT; ++t) {
       if (!a_ok[t]) continue;
       OT* dst = out + orow[t] * ldo + c;
       if (sizeof(OT) == 4) {
@@ -512,16 +512,17 @@ __global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
   }
 }
 
-// bfloat16 operands, tiles of 64 slots, bfloat16 or float32 out.  Refuses (MGPT_ERR_BAD_SHAPE) inner
+// bfloat16 operands, tiles of 64 or 16 slots, bfloat16 or float32 out.  Refuses (MGPT_ERR_BAD_SHAPE) inner
 // sizes that are no multiple of 8, outputs that are no multiple of 4 and unaligned rows or bases;
 // the caller then takes mgpt_grouped_linear.
 extern "C" int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_rows, const void* w, long w_stride,
                                         const int* tile_expert, const int* slot_token, void* out, int out_dtype,
-                                        long ldo, const int* out_rows, int n_tiles, int n_out, int k_dim,
+                                        long ldo, const int* out_rows, int n_tiles, int tile_rows, int n_out, int k_dim,
                                         hipStream_t stream) {
   if (n_tiles == 0 || n_out == 0) return MGPT_OK;
   if (!a || !w || !tile_expert || !slot_token || !out) return MGPT_ERR_NULL;
-  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out) return MGPT_ERR_BAD_SHAPE;
+  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out || (tile_rows != 16 && tile_rows != 64))
+    return MGPT_ERR_BAD_SHAPE;
   const int out_align = out_dtype == MGPT_F32 ? 15 : 7;
   if ((k_dim & 7) || (n_out & 3) || (lda & 7) || (ldo & 3) || (w_stride & 7) || (((size_t)a | (size_t)w) & 15) ||
       (((size_t)out) & out_align))
@@ -529,15 +530,19 @@ extern "C" int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_ro
   if (n_tiles > 65535) return MGPT_ERR_TOO_LARGE;
   // wide outputs: a wave takes 64 columns; narrow ones 16, so that a tile still gives several workgroups
   // ... and so do few tiles (a decode step): more workgroups then walk the inner size side by side
-  const bool wide = n_out >= 512 && n_tiles >= 64;
+  const bool wide = tile_rows == 64 && n_out >= 512 && n_tiles >= 64;
   dim3 grid((n_out + (wide ? 255 : 63)) / (wide ? 256 : 64), n_tiles), block(256);
-#define GM_LAUNCH(OT, NJ)                                                                                     \
-  hipLaunchKernelGGL((grouped_linear_mfma_kernel<OT, NJ>), grid, block, 0, stream, (const bf16_t*)a, lda,     \
+#define GM_LAUNCH(OT, NJ, NT)                                                                                 \
+  hipLaunchKernelGGL((grouped_linear_mfma_kernel<OT, NJ, NT>), grid, block, 0, stream, (const bf16_t*)a, lda, \
                      a_rows, (const bf16_t*)w, w_stride, tile_expert, slot_token, (OT*)out, ldo, out_rows,    \
                      n_out, k_dim)
-  if (out_dtype == MGPT_F32) { if (wide) GM_LAUNCH(float, 4); else GM_LAUNCH(float, 1); }
-  else if (out_dtype == MGPT_BF16) { if (wide) GM_LAUNCH(bf16_t, 4); else GM_LAUNCH(bf16_t, 1); }
-  else return MGPT_ERR_BAD_DTYPE;
+  if (out_dtype == MGPT_F32) {
+    if (tile_rows == 16) GM_LAUNCH(float, 1, 1); else if (wide) GM_LAUNCH(float, 4, 4); else GM_LAUNCH(float, 1, 4);
+  } else if (out_dtype == MGPT_BF16) {
+    if (tile_rows == 16) GM_LAUNCH(bf16_t, 1, 1); else if (wide) GM_LAUNCH(bf16_t, 4, 4); else GM_LAUNCH(bf16_t, 1, 4);
+  } else {
+    return MGPT_ERR_BAD_DTYPE;
+  }
 #undef GM_LAUNCH
   return mgpt_last_error();
 }

@@ -146,7 +146,7 @@ int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, const void* 
     int tile_rows, int n_out, int k_dim, int dtype, hipStream_t stream);
 int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_rows, const void* w, long w_stride, const int*
     tile_expert, const int* slot_token, void* out, int out_dtype, long ldo, const int* out_rows, int n_tiles,
-    int n_out, int k_dim, hipStream_t stream);
+    int tile_rows, int n_out, int k_dim, hipStream_t stream);
 int mgpt_expert_combine(const float* pair_out, const int* pair_slot, const int* q_req, float* y, int n_rows, int
     width, int top, float weight, hipStream_t stream);
 // rms_norm.hip

@@ -1169,12 +1169,12 @@ def grouped_linear(a: torch.Tensor, a_rows: Optional[torch.Tensor], w: torch.Ten
     for t in (a_rows, out_rows):
         if t is not None:
             _need_i32("row index", t, n_slots)
-    if fast and tile == 64 and a.dtype == torch.bfloat16:
+    if fast and tile in (16, 64) and a.dtype == torch.bfloat16:
         # the MFMA kernel; it refuses sizes and alignments that its 16-byte loads do not take
         rc = library.kernels().mgpt_grouped_linear_mfma(_ptr(a), a.stride(0), _ptr(a_rows), _ptr(w), w.stride(0),
                                                         _ptr(tile_expert), _ptr(slot_token), _ptr(out),
                                                         _dtype_code(out), out.stride(0), _ptr(out_rows),
-                                                        n_slots // tile, n_out, k_dim, _stream())
+                                                        n_slots // tile, tile, n_out, k_dim, _stream())
         if rc != -2:
             _check(rc, "grouped_linear_mfma")
             return

@@ -169,7 +169,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_gather_rows": [P, L, P, P, L, I, I, P],
         "mgpt_linear_mfma_grouped": [P, L, P, L, P, P, I, P, I, L, I, I, I, P],
         "mgpt_grouped_linear": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, I, I, P],
-        "mgpt_grouped_linear_mfma": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, P],
+        "mgpt_grouped_linear_mfma": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, I, P],
         "mgpt_expert_combine": [P, P, P, P, I, I, I, F, P],
         "mgpt_router_topk": [P, I, L, P, I, P, I, I, I, I, I, P, P, P],
         "mgpt_gather_scale_rows": [P, I, L, P, P, P, P, L, I, I, P],

@@ -206,8 +206,10 @@ class TableExperts(FeedForward):
         if fast and n * self.top >= self.TILED_FROM_PAIRS and self.width % 16 == 0 and self.hidden % 16 == 0 \
                 and self._forward_tiled(ctx, hn, x, n, ids, table, pair_weight, combine_weight):
             return
-        # tiles of 64 slots for the MFMA kernel of few rows, of 16 for the general one
-        tile = 64 if fast else 16
+        # tiles of 64 slots for the MFMA kernel of few rows, of 16 for the general one, and for the MFMA kernel too
+        # where an expert gets 16 pairs at most on average (a decode step): a tile's empty slots are loaded and
+        # multiplied like the used ones
+        tile = 64 if fast and n * self.top > 16 * self.n_experts else 16
         slots = kernels.expert_slots(n, self.top, self.n_experts, tile)
         slot_token = ws.get("expert_slot_token", slots, 1, torch.int32).view(-1)
         slot_pair = ws.get("expert_slot_pair", slots, 1, torch.int32).view(-1)

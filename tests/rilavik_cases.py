@@ -76,7 +76,7 @@ RAW: Dict[str, dict] = {
     "B": {"architecture": "Rilavik", "vocab": 77, "width": 96, "norm": {"eps": 1e-6},
           "layers": [
               layer("gla", gla(1, 64, 64, 1.0), moe(2, 1, 64)),
-              layer("parallel", parallel(left(2, 2, 64, 64, 0.125, rot=_rot(64, 1e6, 8.0)),
+              layer("parallel", parallel(left(2, 2, 64, 64, 0.125, rot=_rot(64, 3e5, 6.0)),
                                          right(3, 32, 64, 3, 5, 3), 0.5, 0.5), moe(9, 2, 40)),
               layer("parallel", parallel(left(1, 1, 64, 32, 0.125, conv=4, window=100, rot=_rot(32, 50000.0, 4.0)),
                                          right(1, 128, 128, 1, 4, 4), 1.5, 0.25), None)]},
