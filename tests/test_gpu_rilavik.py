@@ -8,6 +8,9 @@ generation through LLMEngine."""
 
 import json
 import math
+import os
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -600,3 +603,45 @@ def test_generation_with_evictions_recomputes_the_state(tmp_path_factory):
     got = tight.generate(prompts, SamplingParams(max_tokens=24, temperature=0.0))
     assert got == want
     assert tight.stats()["num_preemptions"] > 0
+
+
+def test_the_command_line_and_seeded_sampling(tmp_path_factory):
+    """`python -m mini_gpt_inference_amd.generate` on a Rilavik folder: the architecture is found by config.json,
+    greedy tokens are the plain implementation's; sampling with a seed through the engine gives the same tokens
+    whatever the batch a request runs in."""
+    folder = _folder(tmp_path_factory, "D")
+    cfg, w = P.read_model_folder(folder)
+    prompt = [5, 17, 3, 20]
+    want = P.greedy(cfg, w, prompt, 6)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-m", "mini_gpt_inference_amd.generate", "--model", folder,
+                           "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "6", "--temperature", "0",
+                           "--dtype", "float32", "--kv-block-size", "4", "--num-kv-blocks", "32"],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "Rilavik" in proc.stdout
+    line = next(l for l in proc.stdout.splitlines() if l.startswith("sample:"))
+    assert [int(t) for t in line.split()[1:]] == want
+    rng = np.random.default_rng(4)
+    prompts = [helpers.random_ids(rng, cases.RAW["D"]["vocab"], n) for n in (6, 13, 4)]
+    params = [SamplingParams(max_tokens=12, temperature=0.9, top_k=10, seed=7 + i) for i in range(3)]
+    together = LLMEngine.from_folder(folder, EngineConfig(block_size=4, num_blocks=64, max_batch_size=4, dtype="float32"))
+    got = together.generate(prompts, params)
+    for prompt, sp, tokens in zip(prompts, params, got):
+        alone = LLMEngine.from_folder(folder, EngineConfig(block_size=16, num_blocks=16, max_batch_size=1, dtype="float32"))
+        assert alone.generate([prompt], sp) == [tokens]
+
+
+def test_heads_larger_than_the_chunked_form_takes():
+    """Head sizes over 128: the chunked form says no and launches nothing, the token-by-token kernel takes them."""
+    mode, H, G, D, E = "channel_sigmoid", 1, 1, 160, 24
+    z, a, offs, extra, want = _state_case(mode, H, G, D, E, "float32", 3, 2.0)
+    state = torch.full((6, H * D * E), float("nan"), device=DEV)
+    rows, cu, pos, _, slots = _step_arrays(WHOLE[0])
+    out = torch.full((len(rows), H * E), 9.0, device=DEV)
+    assert not kernels.gated_state_chunked(z[rows].to(DEV), offs["q_off"], offs["k_off"], offs["v_off"], H, G, D, E,
+                                           a[rows].to(DEV), offs["a_off"], mode, state, slots, cu, len(WHOLE[0]) + 1,
+                                           len(rows), pos, torch.zeros(len(rows), 3 * H * D, device=DEV), out, **extra)
+    assert (out == 9.0).all() and torch.isnan(state).all()
+    got = _run_state(PORTIONS, False, mode, H, G, D, E, z, a, offs, extra, state)
+    helpers.assert_close(got, want, "float32", "heads of 160")
