@@ -345,6 +345,10 @@ class DecoderModel:
                 else:
                     bindings[role] = CacheBinding("none")
             run_bindings.append(bindings)
+        if not groups:
+            # a model that keeps no keys and values (state mixers only): one group without pools, so that the
+            # page tables, which also say how far every request has come, still have something to count in
+            groups.append(CacheGroupSpec(1, 1, 0, 0, False))
         return CacheLayout(groups, state_numels, run_bindings)
 
     @property

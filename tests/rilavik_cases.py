@@ -89,15 +89,20 @@ RAW: Dict[str, dict] = {
               layer("parallel", parallel(left(4, 2, 12, 20, 0.5, conv=2, window=16, rot=_rot(6, 200.0, 1.5)),
                                          right(6, 4, 12, 2, 3, 3), 1.0, 1.0), moe(7, 3, 72)),
               layer("gla", gla(2, 36, 20, 2.5), None)]},
-    # parallel layers only, then gla layers only
+    # a parallel layer, then a gla layer
     "D": {"architecture": "Rilavik", "vocab": 33, "width": 32, "norm": {"eps": 1e-5},
           "layers": [
               layer("parallel", parallel(left(2, 1, 16, 16, 0.25, conv=4, window=33, rot=_rot(16, 10000.0)),
                                          right(2, 16, 16, 1, 4, 1), 0.8, 0.6), moe(3, 1, 32)),
               layer("gla", gla(2, 16, 16, 8.0), moe(6, 2, 16))]},
+    # gla layers only: no keys and values, no pages with anything in them
+    "E": {"architecture": "Rilavik", "vocab": 45, "width": 48, "norm": {"eps": 1e-5},
+          "layers": [
+              layer("gla", gla(2, 24, 16, 4.0), moe(4, 2, 24)),
+              layer("gla", gla(3, 16, 32, 32.0), None)]},
 }
-SEEDS = {"A": 21, "B": 22, "C": 23, "D": 24}
-DECAY_RANKS = {"A": 8, "B": 16, "C": 5, "D": 4}
+SEEDS = {"A": 21, "B": 22, "C": 23, "D": 24, "E": 25}
+DECAY_RANKS = {"A": 8, "B": 16, "C": 5, "D": 4, "E": 6}
 STD_SCALE = 1.5
 
 

@@ -327,7 +327,8 @@ def test_a_key_just_inside_and_just_outside_the_window(dtype, D, window):
 
 
 # ---------------------------------------------------------------- the model through the step function
-LENGTHS = {"A": [5, 70, 23, 41, 2, 64, 37], "B": [1, 9, 33, 17, 110], "C": [40, 3, 64, 21], "D": [75, 12, 30, 6, 49]}
+LENGTHS = {"A": [5, 70, 23, 41, 2, 64, 37], "B": [1, 9, 33, 17, 110], "C": [40, 3, 64, 21], "D": [75, 12, 30, 6, 49],
+           "E": [33, 4, 70, 18, 2]}
 _folders, _plain, _twin = {}, {}, {}
 
 
@@ -559,7 +560,7 @@ def test_sharp_attention_at_the_windows_edge_prefill_and_decoding(tmp_path, dtyp
         _check(folder, "sharp", dtype, "a", ids, got["a"], want, f"sharp {dtype} {way}")
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "E"])
 def test_greedy_generation_through_the_engine(tmp_path_factory, name):
     folder = _folder(tmp_path_factory, name)
     cfg, w = P.read_model_folder(folder)

@@ -277,3 +277,13 @@ def test_no_convolution_no_rotation_no_window_leave_their_tensors_and_state_out(
     assert "l1.mix.left.q.conv" not in wanted and "l2.mix.left.q.conv" in wanted
     kv = [p.cache_need() for layer in model.layers for r, p in layer.parts.items() if r == "mixer0"]
     assert [(n.window, n.state_numel) for n in kv] == [(0, 0), (100, 3 * 3 * 64)]
+
+
+def test_a_model_of_state_mixers_only_still_has_a_group_of_pages():
+    """No mixer keeps keys and values: the layout holds one group without pools, whose page tables only count
+    how far every request has come."""
+    model = DecoderModel(rilavik.model_spec(cases.config("E")))
+    layout = model.cache_layout
+    assert [(g.n_pools, g.window) for g in layout.groups] == [(0, 0)]
+    assert [b.kind for run in layout.run_bindings for b in run.values()] == ["state", "state"]
+    assert layout.state_numels == [2 * 24 * 16, 3 * 16 * 32]
