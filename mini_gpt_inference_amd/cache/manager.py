@@ -17,6 +17,7 @@ class GroupGeometry:
     page_size: int
     num_pages: int
     window: int = 0
+    keep_first: int = 0     # with a window: the first positions that every query still sees; their pages are kept
 
 
 class CacheError(RuntimeError):
@@ -34,14 +35,15 @@ def plan_group_pages(groups, page_size: int, num_blocks: int, kv_cache_bytes, it
     the same number of full-length requests: a group's page costs n_pools * 2 (1 where keys and values
     are one joint tensor) * n_kv_head * page_size
     * head_dim * itemsize bytes, and a full-length request holds its whole span in a group that
-    keeps all keys but only a window (and the page being written) in one that keeps a window."""
+    keeps all keys but only a window (and the page being written, and the first positions that the
+    window keeps) in one that keeps a window."""
     if kv_cache_bytes is None:
         return [int(num_blocks)] * len(groups)
     span_all = int(max_positions) if max_positions else NOMINAL_SPAN
     page_bytes, pages_per_request = [], []
     for g in groups:
         page_bytes.append(g.n_pools * (1 if getattr(g, "joint", False) else 2) * g.n_kv_head * page_size * g.head_dim * itemsize)
-        span = min(g.window + page_size, span_all) if g.window else span_all
+        span = min(g.window + page_size + getattr(g, "keep_first", 0), span_all) if g.window else span_all
         pages_per_request.append(-(-span // page_size))
     per_request = sum(b * n for b, n in zip(page_bytes, pages_per_request))
     if per_request <= 0:
@@ -71,7 +73,8 @@ class CacheManager:
         arr = lambda vals: (ctypes.c_int * n)(*vals)
         self._h = self._lib.mgpt_cache_create(n, arr([g.page_size for g in self.groups]),
                                               arr([g.num_pages for g in self.groups]),
-                                              arr([g.window for g in self.groups]), self.max_requests)
+                                              arr([g.window for g in self.groups]),
+                                              arr([g.keep_first for g in self.groups]), self.max_requests)
         if not self._h:
             raise CacheError(library.host_error())
 

@@ -12,7 +12,9 @@
 // absolute key position).  Inside a chunk each lane scores one key with 16-byte loads of its
 // row; then the lanes turn to the head's channels and add the chunk's values.  The four
 // partial results (max, sum, weighted values) are merged through LDS in wave order.
-// Slots outside the visible range are never loaded.
+// Slots outside the visible range are never loaded.  With `keep_first` > 0 a query behind a window also sees
+// the keys at positions below keep_first; with `score_bias` a visible key's weight is
+// sigmoid(score + score_bias[head]) and nothing is normalised.
 #include "common.h"
 #include "launchers.h"
 
@@ -25,7 +27,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
     int n_kv_head, int head_dim, int page_size, float scale, int window, const float* __restrict__ sinks,
-    float softcap, const bf16_t* __restrict__ gate, long ldg) {
+    float softcap, const bf16_t* __restrict__ gate, long ldg, int keep_first, const float* __restrict__ score_bias) {
   __shared__ float q_s[AD_MAX_DPL * 64];
   __shared__ float p_s[AD_WAVES][64];
   __shared__ int page_s[AD_WAVES][64];
@@ -54,10 +56,16 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
 #pragma unroll
   for (int i = 0; i < AD_MAX_DPL; ++i) acc[i] = 0.f;
 
+  const bool weigh = score_bias != nullptr;   // sigmoid weights, no softmax
+  const float bias = weigh ? score_bias[h] : 0.f;
+  // the chunks of the kept first keys (those before the window's first chunk), then the window's
   const int first_chunk = kv_begin / 64;
-  for (int c0 = (first_chunk + wave) * 64; c0 < kv_end; c0 += 64 * AD_WAVES) {
+  const int kept_chunks = keep_first > 0 ? ((keep_first + 63) / 64 < first_chunk ? (keep_first + 63) / 64 : first_chunk) : 0;
+  const int n_chunks = kept_chunks + (kv_end + 63) / 64 - first_chunk;
+  for (int ci = wave; ci < n_chunks; ci += AD_WAVES) {
+    const int c0 = (ci < kept_chunks ? ci : first_chunk + ci - kept_chunks) * 64;
     const int j = c0 + lane;
-    const bool valid = (j >= kv_begin) && (j < kv_end);
+    const bool valid = (j >= kv_begin || j < keep_first) && (j < kv_end);
     float s = -INFINITY;
     int page = -1;
     if (valid) {
@@ -76,16 +84,22 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
       }
       s = softcap > 0.f ? softcap * tanh_fast(dot * __builtin_amdgcn_rcpf(softcap)) : dot;
     }
-    const float m_new = fmaxf(m, wave_max(s));
-    const float p = valid ? __expf(s - m_new) : 0.f;
-    const float alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
-    l = l * alpha + wave_sum(p);
-    m = m_new;
+    float p = 0.f, alpha = 1.f;
+    if (weigh) {
+      if (valid) p = __builtin_amdgcn_rcpf(1.0f + __expf(-(s + bias)));
+      m = 0.f;
+    } else {
+      const float m_new = fmaxf(m, wave_max(s));
+      p = valid ? __expf(s - m_new) : 0.f;
+      alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
+      l = l * alpha + wave_sum(p);
+      m = m_new;
+    }
     // p_s / page_s rows are private to the wave; a wave runs in lockstep, so no barrier is needed
     p_s[wave][lane] = p;
     page_s[wave][lane] = page;
     __builtin_amdgcn_wave_barrier();
-    const int j_lo = (kv_begin > c0 ? kv_begin : c0) - c0;
+    const int j_lo = ((kv_begin > c0 && c0 >= keep_first) ? kv_begin : c0) - c0;
     const int j_hi = (kv_end < c0 + 64 ? kv_end : c0 + 64) - c0;
 #pragma unroll
     for (int i = 0; i < AD_MAX_DPL; ++i) {
@@ -94,6 +108,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
         float a = acc[i] * alpha;
 #pragma unroll 8
         for (int jj = j_lo; jj < j_hi; ++jj) {
+          if (page_s[wave][jj] < 0) continue;   // between the kept first keys and the window
           const int off = (c0 + jj) % page_size;
           const bf16_t* vr = vpool + (((long)page_s[wave][jj] * n_kv_head + hk) * page_size + off) * (long)head_dim;
           a = fmaf(p_s[wave][jj], bf16_to_float(vr[d]), a);
@@ -127,7 +142,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
       f[w] = (m_s[w] == -INFINITY) ? 0.f : __expf(m_s[w] - mx);
       lt += l_s[w] * f[w];
     }
-    float inv = 1.0f / lt;
+    float inv = weigh ? 1.0f : 1.0f / lt;
     if (gate) inv *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)n * ldg + h])));   // sigmoid gate of the head
 #pragma unroll
     for (int i = 0; i < AD_MAX_DPL; ++i) {
@@ -145,17 +160,20 @@ extern "C" int mgpt_paged_attention_split_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
+    const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const float* score_bias,
+    hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || head_dim <= 0 ||
-      head_dim > AD_MAX_DPL * 64 || (head_dim % 8) != 0 || page_size <= 0 || max_blocks <= 0 || window < 0)
+      head_dim > AD_MAX_DPL * 64 || (head_dim % 8) != 0 || page_size <= 0 || max_blocks <= 0 || window < 0 ||
+      keep_first < 0 || (score_bias && (sinks || softcap > 0.f)))
     return MGPT_ERR_BAD_SHAPE;
+  if (window == 0) keep_first = 0;
   if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
   hipLaunchKernelGGL(paged_attention_split_kernel, dim3(n_tokens, n_head), dim3(256), 0, stream,
                      (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,
                      block_tables, max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim,
-                     page_size, scale, window, sinks, softcap, (const bf16_t*)gate, ldg);
+                     page_size, scale, window, sinks, softcap, (const bf16_t*)gate, ldg, keep_first, score_bias);
   return mgpt_last_error();
 }
 
@@ -172,7 +190,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
     int n_kv_head, int page_size, float scale, int window, const float* __restrict__ sinks, float softcap,
-    const bf16_t* __restrict__ gate, long ldg) {
+    const bf16_t* __restrict__ gate, long ldg, int keep_first, const float* __restrict__ score_bias) {
   constexpr int LPK = D / 8;     // lanes per key
   constexpr int KPI = 64 / LPK;  // keys per load instruction
   __shared__ float m_s[AD_WAVES], l_s[AD_WAVES];
@@ -208,14 +226,19 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
 
+  const bool weigh = score_bias != nullptr;   // sigmoid weights, no softmax
+  const float bias = weigh ? score_bias[h] : 0.f;
   const int first_chunk = kv_begin / 64;
-  for (int c0 = (first_chunk + wave) * 64; c0 < kv_end; c0 += 64 * AD_WAVES) {
+  const int kept_chunks = keep_first > 0 ? ((keep_first + 63) / 64 < first_chunk ? (keep_first + 63) / 64 : first_chunk) : 0;
+  const int n_chunks = kept_chunks + (kv_end + 63) / 64 - first_chunk;
+  for (int ci = wave; ci < n_chunks; ci += AD_WAVES) {
+    const int c0 = (ci < kept_chunks ? ci : first_chunk + ci - kept_chunks) * 64;
     long base[LPK];
     bool valid[LPK];
 #pragma unroll
     for (int i = 0; i < LPK; ++i) {
       const int j = c0 + i * KPI + sub;
-      valid[i] = (j >= kv_begin) && (j < kv_end);
+      valid[i] = (j >= kv_begin || j < keep_first) && (j < kv_end);
       base[i] = 0;
       if (valid[i]) {
         const int page = bt[j / page_size];
@@ -245,14 +268,14 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
       s[i] = valid[i] ? dot : -INFINITY;
       cmax = fmaxf(cmax, s[i]);
     }
-    const float m_new = fmaxf(m, wave_max(cmax));
-    const float alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
+    const float m_new = weigh ? 0.f : fmaxf(m, wave_max(cmax));
+    const float alpha = weigh ? 1.f : ((m == -INFINITY) ? 0.f : __expf(m - m_new));
     float psum = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] *= alpha;
 #pragma unroll
     for (int i = 0; i < LPK; ++i) {
-      const float p = valid[i] ? __expf(s[i] - m_new) : 0.f;
+      const float p = !valid[i] ? 0.f : (weigh ? __builtin_amdgcn_rcpf(1.0f + __expf(-(s[i] + bias))) : __expf(s[i] - m_new));
       psum += p;
       const unsigned int w[4] = {vraw[i].x, vraw[i].y, vraw[i].z, vraw[i].w};
 #pragma unroll
@@ -292,7 +315,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
       lt += l_s[w] * f;
       a += acc_s[w][tid] * f;
     }
-    float res = a / lt;
+    float res = weigh ? a : a / lt;
     if (gate) res *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)n * ldg + h])));
     out[(long)n * ldo + (long)h * D + tid] = float_to_bf16(res);
   }
@@ -302,19 +325,21 @@ extern "C" int mgpt_paged_attention_split_fast_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
+    const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const float* score_bias,
+    hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
-      max_blocks <= 0 || window < 0 || (ldq % 8) != 0)
+      max_blocks <= 0 || window < 0 || (ldq % 8) != 0 || keep_first < 0 || (score_bias && (sinks || softcap > 0.f)))
     return MGPT_ERR_BAD_SHAPE;
+  if (window == 0) keep_first = 0;
   if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
   dim3 grid(n_tokens, n_head), block(256);
 #define AD_LAUNCH(DD)                                                                                   \
   hipLaunchKernelGGL(paged_attention_split_fast_kernel<DD>, grid, block, 0, stream, (const bf16_t*)q, ldq, \
                      (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,       \
                      max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window, sinks, softcap, \
-                     (const bf16_t*)gate, ldg)
+                     (const bf16_t*)gate, ldg, keep_first, score_bias)
   switch (head_dim) {
     case 16: AD_LAUNCH(16); break;
     case 32: AD_LAUNCH(32); break;

@@ -19,6 +19,9 @@
 //    then the four rows' values through scalar registers); the weighted sum of values again with
 //    v_dot2_f32_bf16, two keys at a time, the weights rounded to bfloat16 as the tile kernel
 //    for prompts does;
+//  * with `keep_first` > 0 a query behind a window also sees the keys at positions below keep_first: the first
+//    pass then starts at key 0 and the passes behind the kept keys go on at the window's first chunk; with
+//    `score_bias` a visible key's weight is sigmoid(score + score_bias[head]) and nothing is normalised;
 //  * the waves' partial results (maximum, sum, weighted values per key subgroup) are merged
 //    through LDS once, in a fixed order.
 #include "common.h"
@@ -70,7 +73,7 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ q_req, const int* __restrict__ cu_q, int n_head, int n_kv_head, int page_shift,
     int num_pages, unsigned int page_bytes, float scale_log2e, int window, const float* __restrict__ sinks,
-    float cap_log2e, const bf16_t* __restrict__ gate, long ldg) {
+    float cap_log2e, const bf16_t* __restrict__ gate, long ldg, int keep_first, const float* __restrict__ score_bias) {
   constexpr int LPK = D / 8;     // lanes per key
   constexpr int KPI = 64 / LPK;  // keys per load instruction
   constexpr int ROWS = AW_WAVES * KPI;      // partial results: one per (key subgroup, wave)
@@ -101,15 +104,19 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
   int first_chunk = 0;
   if (window > 0) first_chunk = (qpos - window + 1 > 0 ? qpos - window + 1 : 0) / 64;  // waits for qpos
   const int* bt = block_tables + (long)r * max_blocks;
+  const bool weigh = score_bias != nullptr;   // sigmoid weights, no softmax
+  const float bias_log2e = weigh ? score_bias[h] * 1.4426950408889634f : 0.f;
 
   float m = -INFINITY, l = 0.f;
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
 
-  int c_base = first_chunk * 64;
+  int c_base = keep_first > 0 ? 0 : first_chunk * 64;
   int kv_end = 0, kv_begin = 0;
   do {
+    // a pass that lies wholly between the kept first keys and the window's first chunk: on to that chunk
+    if (c_base >= keep_first && c_base < first_chunk * 64) c_base = first_chunk * 64;
     const int c0 = c_base + wave * 64;
     const int page_mask = (1 << page_shift) - 1;
     int page[LPK];
@@ -122,7 +129,7 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
     kv_begin = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
     c_base += 64 * AW_WAVES;
     // a chunk without a visible key costs its wave nothing more (the same decision in all lanes)
-    if (__builtin_amdgcn_readfirstlane((c0 >= kv_end) | (c0 + 64 <= kv_begin))) continue;
+    if (__builtin_amdgcn_readfirstlane((c0 >= kv_end) | ((c0 + 64 <= kv_begin) & (c0 >= keep_first)))) continue;
     // ---- second round trip: keys and values of this wave's chunk.  Every lane loads (a masked
     // key reads the pool's first row instead and is zeroed afterwards), so that no branch stands
     // between the loads.  Offsets are 32-bit byte offsets from the pools' bases.
@@ -132,7 +139,7 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
 #pragma unroll
     for (int i = 0; i < LPK; ++i) {
       const int j = c0 + i * KPI + sub;
-      valid[i] = (j >= kv_begin) && (j < kv_end);
+      valid[i] = (j >= kv_begin || j < keep_first) && (j < kv_end);
       const bool follow = valid[i] && (unsigned int)page[i] < (unsigned int)num_pages;
       const unsigned int row_off = ((unsigned int)page[i] * page_bytes) + (unsigned int)(j & page_mask) * (D * 2u);
       const unsigned int off = follow ? row_off + lane_off : 0u;
@@ -156,7 +163,7 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
       s[i] = valid[i] ? dot : -INFINITY;
       cmax = fmaxf(cmax, s[i]);
     }
-    const float m_new = fmaxf(m, aw_wave_max(cmax));
+    const float m_new = weigh ? 0.f : fmaxf(m, aw_wave_max(cmax));
     if (m_new != -INFINITY) {  // the same in all lanes; false only while the wave has seen no key
       const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // m = -inf: 0
       l *= alpha;
@@ -165,7 +172,9 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
       m = m_new;
 #pragma unroll
       for (int i = 0; i < LPK; i += 2) {
-        const float pa = __builtin_amdgcn_exp2f(s[i] - m_new), pb = __builtin_amdgcn_exp2f(s[i + 1] - m_new);  // a masked key: exp2(-inf) = 0
+        // a masked key: exp2(-inf) = 0, and 1 / (1 + exp2(inf)) = 0
+        const float pa = weigh ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-(s[i] + bias_log2e))) : __builtin_amdgcn_exp2f(s[i] - m_new);
+        const float pb = weigh ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-(s[i + 1] + bias_log2e))) : __builtin_amdgcn_exp2f(s[i + 1] - m_new);
         l += pa + pb;
         const unsigned int pp = pack_bf16x2(pa, pb);
         const unsigned int va[4] = {vraw[i].x, vraw[i].y, vraw[i].z, vraw[i].w};
@@ -225,7 +234,7 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
       for (int w = 0; w < AW_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
       lt += __builtin_amdgcn_exp2f(sink - mx);
     }
-    float res = a / lt;
+    float res = score_bias ? a : a / lt;
     if (gate) res *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)n * ldg + h])));   // sigmoid gate of the head
     out[(long)n * ldo + (long)h * D + tid] = float_to_bf16(res);
   }
@@ -241,12 +250,15 @@ extern "C" int mgpt_paged_attention_decode_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* positions, const int* q_req, const int* cu_q,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, int num_pages, float scale, int window,
-    int identity, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
+    int identity, const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const float* score_bias,
+    hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !positions || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
-      max_blocks <= 0 || num_pages <= 0 || window < 0 || (ldq % 8) != 0 || (identity && cu_q))
+      max_blocks <= 0 || num_pages <= 0 || window < 0 || (ldq % 8) != 0 || (identity && cu_q) || keep_first < 0 ||
+      (score_bias && (sinks || softcap > 0.f)))
     return MGPT_ERR_BAD_SHAPE;
+  if (window == 0) keep_first = 0;
   if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
   int page_shift = -1;
   for (int s = 0; s < 30; ++s)
@@ -263,7 +275,7 @@ extern "C" int mgpt_paged_attention_decode_bf16(
                      (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,          \
                      max_blocks, positions, q_req, cu_q, n_head, n_kv_head, page_shift, num_pages, page_bytes, \
                      scale_log2e, window, sinks, softcap > 0.f ? softcap * 1.4426950408889634f : 0.f, \
-                     (const bf16_t*)gate, ldg)
+                     (const bf16_t*)gate, ldg, keep_first, score_bias)
 #define AW_LAUNCH(DD)              \
   do {                             \
     if (identity) AW_LAUNCH2(DD, true); \

@@ -11,6 +11,9 @@
 // softmax over keys in 32-bit (with `sinks`, one more term exp(sinks[head]) in its denominator that
 // has no value; with `softcap` > 0 every score becomes softcap * tanh(score / softcap) first; with `gate`
 // a head's output is multiplied by sigmoid(gate[token][head]));
+// with `keep_first` > 0 a query behind a window also sees the keys at positions below keep_first; with
+// `score_bias` (a number per head) there is no softmax: a visible key's weight is
+// sigmoid(score + score_bias[head]), and the weights are not normalised;
 // y = P v (reference: src/minigpt_infer/model.py:61-87,
 // the rule col <= cache_len + row of src/minigpt_infer/batch.py:202-227).
 //
@@ -73,7 +76,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ cu_q, const int* __restrict__ seq_lens, const int* __restrict__ q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* __restrict__ sinks, float softcap, const T* __restrict__ gate, long ldg) {
+    const float* __restrict__ sinks, float softcap, const T* __restrict__ gate, long ldg, int keep_first,
+    const float* __restrict__ score_bias) {
   __shared__ float q_s[MAX_DPL * MGPT_WAVE];
   __shared__ float p_s[MGPT_WAVE];
   __shared__ int page_s[MGPT_WAVE];
@@ -99,9 +103,15 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
 #pragma unroll
   for (int i = 0; i < MAX_DPL; ++i) acc[i] = 0.f;
 
-  for (int c0 = (kv_begin / MGPT_WAVE) * MGPT_WAVE; c0 < kv_end; c0 += MGPT_WAVE) {
+  const bool weigh = score_bias != nullptr;   // sigmoid weights, no softmax
+  const float bias = weigh ? score_bias[h] : 0.f;
+  for (int c0 = 0; c0 < kv_end; c0 += MGPT_WAVE) {
+    if (c0 + MGPT_WAVE <= kv_begin && c0 >= keep_first) {   // behind the kept first keys, before the window: on to the window's chunk
+      c0 = (kv_begin / MGPT_WAVE) * MGPT_WAVE - MGPT_WAVE;
+      continue;
+    }
     const int j = c0 + lane;
-    const bool valid = (j >= kv_begin) && (j < kv_end);
+    const bool valid = (j >= kv_begin || j < keep_first) && (j < kv_end);
     float s = -INFINITY;
     int page = -1;
     if (valid) {
@@ -113,24 +123,28 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
       s = dot * scale;
       if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
-    const float m_new = fmaxf(m, wave_max(s));
-    float p = 0.f;
-    if (valid) p = FAST_EXP ? __expf(s - m_new) : expf(s - m_new);
-    const float alpha = (m == -INFINITY) ? 0.f : (FAST_EXP ? __expf(m - m_new) : expf(m - m_new));
-    l = l * alpha + wave_sum(p);
-    m = m_new;
+    float p = 0.f, alpha = 1.f;
+    if (weigh) {
+      if (valid) p = 1.0f / (1.0f + (FAST_EXP ? __expf(-(s + bias)) : expf(-(s + bias))));
+    } else {
+      const float m_new = fmaxf(m, wave_max(s));
+      if (valid) p = FAST_EXP ? __expf(s - m_new) : expf(s - m_new);
+      alpha = (m == -INFINITY) ? 0.f : (FAST_EXP ? __expf(m - m_new) : expf(m - m_new));
+      l = l * alpha + wave_sum(p);
+      m = m_new;
+    }
     __syncthreads();  // previous chunk's readers of p_s / page_s are done
     p_s[lane] = p;
     page_s[lane] = page;
     __syncthreads();
-    const int j_lo = (kv_begin > c0 ? kv_begin : c0) - c0;
     const int j_hi = (kv_end < c0 + MGPT_WAVE ? kv_end : c0 + MGPT_WAVE) - c0;
 #pragma unroll
     for (int i = 0; i < MAX_DPL; ++i) {
       const int d = lane + i * MGPT_WAVE;
       if (d < head_dim) {
         float a = acc[i] * alpha;
-        for (int jj = j_lo; jj < j_hi; ++jj) {
+        for (int jj = 0; jj < j_hi; ++jj) {
+          if (page_s[jj] < 0) continue;   // a key that the query does not see
           const int off = (c0 + jj) % page_size;
           const T* vr = vpool + (((long)page_s[jj] * n_kv_head + hk) * page_size + off) * (long)head_dim;
           a = fmaf(p_s[jj], to_float<T>(vr[d]), a);
@@ -148,7 +162,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < MAX_DPL; ++i) acc[i] *= alpha;
   }
-  float inv_l = 1.0f / l;
+  float inv_l = weigh ? 1.0f : 1.0f / l;
   if (gate) {   // the head's output times sigmoid(gate[token][head])
     const float gv = to_float<T>(gate[(long)n * ldg + h]);
     inv_l *= 1.0f / (1.0f + (FAST_EXP ? __expf(-gv) : expf(-gv)));
@@ -167,19 +181,21 @@ extern "C" int mgpt_paged_attention_generic(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    int dtype, int fast_exp, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
+    int dtype, int fast_exp, const float* sinks, float softcap, const void* gate, long ldg, int keep_first,
+    const float* score_bias, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || head_dim <= 0 ||
-      head_dim > MAX_DPL * MGPT_WAVE || page_size <= 0 || max_blocks <= 0 || window < 0)
+      head_dim > MAX_DPL * MGPT_WAVE || page_size <= 0 || max_blocks <= 0 || window < 0 || keep_first < 0 || (score_bias && (sinks || softcap > 0.f)))
     return MGPT_ERR_BAD_SHAPE;
   if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
+  if (window == 0) keep_first = 0;   // every key is seen anyway
   dim3 grid(n_tokens, n_head), block(MGPT_WAVE);
 #define LAUNCH(T, F)                                                                              \
   hipLaunchKernelGGL((paged_attention_generic_kernel<T, F>), grid, block, 0, stream, (const T*)q, ldq, \
                      (T*)out, ldo, (const T*)kpool, (const T*)vpool, block_tables, max_blocks, cu_q,  \
                      seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim, page_size, scale, window, sinks, softcap, \
-                     (const T*)gate, ldg)
+                     (const T*)gate, ldg, keep_first, score_bias)
   if (dtype == MGPT_F32) {
     if (fast_exp) LAUNCH(float, true); else LAUNCH(float, false);
   } else if (dtype == MGPT_BF16) {

@@ -5,6 +5,10 @@
 // with ctx > 0 is the offset-causal case of src/minigpt_infer/batch.py:202-227), scores scaled,
 // softmax and all sums in float32 (src/minigpt_infer/model.py:61-87).
 //
+// With `keep_first` > 0 a query behind a window also sees the keys at positions below keep_first (a tile walks
+// the stretches of those keys first, then the window's); with `score_bias` a visible key's weight is
+// sigmoid(score + score_bias[head]) and nothing is normalised.
+//
 // A workgroup takes 64 consecutive queries of one request and one head, 16 per wave (four waves,
 // or eight in two groups that share the keys between them, see the kernel).  It walks the keys in blocks of 128 (aligned to multiples of 128 of the key position):
 // the block's key and value rows go to LDS as they are, gathered row by row through the block
@@ -65,7 +69,8 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_head, int n_kv_head, int page_size, float scale, int window,
-    int single_below, const float* __restrict__ sinks, float softcap, const bf16_t* __restrict__ gate, long ldg) {
+    int single_below, const float* __restrict__ sinks, float softcap, const bf16_t* __restrict__ gate, long ldg,
+    int keep_first, const float* __restrict__ score_bias) {
   constexpr int THREADS = 256 * G;
   constexpr int SB = PF_KT * G;    // keys staged per step
   // Key and value rows in LDS: as long as the head size where that is a power of two, the 16-byte
@@ -128,7 +133,7 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
 
   // the row index of key j, or -1; the block table entry is the only thing read from memory
   auto lookup = [&](int j) -> int {
-    if (j < kv_begin || j >= kv_end) return -1;
+    if (j >= kv_end || (j < kv_begin && j >= keep_first)) return -1;
     const int pg = j / page_size;
     return (bt[pg] * n_kv_head + hk) * page_size + (j - pg * page_size);
   };
@@ -164,10 +169,15 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
 
   // scores are kept in units of log2(e), so that the exponential is one v_exp_f32 (scale > 0 here)
   const float sc2 = scale * 1.4426950408889634f;
+  const bool weigh = score_bias != nullptr;   // sigmoid weights, no softmax
+  const float bias2 = weigh ? score_bias[h] * 1.4426950408889634f : 0.f;
   const int c_first = (kv_begin / SB) * SB;
-  const int n_steps = (kv_end - c_first + SB - 1) / SB;
+  // the stretches of the kept first keys (those before the window's first stretch), then the window's
+  const int kept_steps = keep_first > 0 ? ((keep_first + SB - 1) / SB < c_first / SB ? (keep_first + SB - 1) / SB : c_first / SB) : 0;
+  const int n_steps = kept_steps + (kv_end - c_first + SB - 1) / SB;
+  auto stretch_start = [&](int step) -> int { return step < kept_steps ? step * SB : c_first + (step - kept_steps) * SB; };
   // the rows of the first three stretches
-  for (int t = tid; t < 3 * SB; t += THREADS) row_tab[t] = lookup(c_first + t);
+  for (int t = tid; t < 3 * SB; t += THREADS) row_tab[t] = lookup(stretch_start(t / SB) + t % SB);
   __syncthreads();
   fetch(0);
   deposit(0);
@@ -175,16 +185,16 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
   __syncthreads();
   for (int b = 0; b < n_steps; ++b) {
     const int buf = b & 1;
-    const int c0 = c_first + b * SB + grp * PF_KT;   // first key of this wave group's half
+    const int c0 = stretch_start(b) + grp * PF_KT;   // first key of this wave group's half
     int row_ahead = -1;
     if (b + 1 < n_steps) {
       deposit(buf ^ 1);   // its readers finished before the last barrier
       if (b + 2 < n_steps) fetch(b + 2);
       // asked for now, written to the table at the end of this step's work
-      if (b + 3 < n_steps && tid < SB) row_ahead = lookup(c_first + (b + 3) * SB + tid);
+      if (b + 3 < n_steps && tid < SB) row_ahead = lookup(stretch_start(b + 3) + tid);
     }
     // a half with no key that the tile sees (past the end, or before a window) is left out
-    if (c0 < kv_end && c0 + PF_KT > kv_begin) {
+    if (c0 < kv_end && (c0 + PF_KT > kv_begin || c0 < keep_first)) {
       const bf16_t* ks = pf_lds + buf * KS_SIZE + grp * PF_KT * KLD;
       const bf16_t* vs = pf_lds + (2 + buf) * KS_SIZE + grp * PF_KT * KLD;
 
@@ -250,14 +260,14 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int key = c0 + kt * 16 + g * 4 + i;
-            const bool see = q_ok && key <= my_pos && key >= kv_begin && (window <= 0 || key > my_pos - window);
+            const bool see = q_ok && key <= my_pos && (window <= 0 || key > my_pos - window || key < keep_first);
             const float v = see ? s[kt][i] : -INFINITY;
             s[kt][i] = v;
             mx = fmaxf(mx, v);
           }
       }
       mx = pf_max_over_rows(mx) * sc2;   // -inf stays -inf
-      const float m_new = fmaxf(m, mx);
+      const float m_new = weigh ? 0.f : fmaxf(m, mx);
       const float alpha = (m == -INFINITY) ? ((m_new == -INFINITY) ? 1.f : 0.f) : __builtin_amdgcn_exp2f(m - m_new);
       const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;   // exp2(-inf - 0) = 0 for masked scores
       float rs = 0.f;
@@ -267,7 +277,9 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
         float p[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt + (i >> 2)][i & 3], sc2, -m_sub));
+          const float e = __builtin_fmaf(s[kt + (i >> 2)][i & 3], sc2, -m_sub);
+          // (a masked score is -inf: exp2(-inf) = 0, and 1 / (1 + exp2(inf)) = 0)
+          p[i] = weigh ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-(e + bias2))) : __builtin_amdgcn_exp2f(e);
           rs += p[i];
         }
         const u32x4_t packed = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
@@ -335,7 +347,7 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
       for (int i = 0; i < 4; ++i) o[dt][i] *= a;
   }
   if (q_ok) {
-    float inv = 1.0f / l;
+    float inv = weigh ? 1.0f : 1.0f / l;
     if (gate)   // the head's output times sigmoid(gate[token][head])
       inv *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)(q_start + my_q) * ldg + h])));
     bf16_t* orow = out + (long)(q_start + my_q) * ldo + (long)h * D;
@@ -360,13 +372,15 @@ extern "C" int mgpt_prefill_attention_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req,
     int max_q_len, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    int single_below, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
+    int single_below, const float* sinks, float softcap, const void* gate, long ldg, int keep_first,
+    const float* score_bias, hipStream_t stream) {
   if (n_req == 0 || max_q_len == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens) return MGPT_ERR_NULL;
   if (n_req < 0 || max_q_len < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 ||
       page_size <= 0 || max_blocks <= 0 || window < 0 || (ldq % 8) != 0 || (ldo % 4) != 0 ||
-      (((size_t)out) & 7) != 0 || !(scale > 0.f))
+      (((size_t)out) & 7) != 0 || !(scale > 0.f) || keep_first < 0 || (score_bias && (sinks || softcap > 0.f)))
     return MGPT_ERR_BAD_SHAPE;
+  if (window == 0) keep_first = 0;
   if (n_req > 65535 || n_head > 65535) return MGPT_ERR_TOO_LARGE;
   dim3 grid((max_q_len + PF_QT - 1) / PF_QT, n_req, n_head);
 #define PF_LAUNCH(DD, GG)                                                                                       \
@@ -384,7 +398,7 @@ extern "C" int mgpt_prefill_attention_bf16(
     hipLaunchKernelGGL((prefill_attention_kernel<DD, GG>), grid, dim3(256 * GG), lds_bytes, stream,             \
                        (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,    \
                        block_tables, max_blocks, cu_q, seq_lens, n_head, n_kv_head, page_size, scale, window,   \
-                       single_below, sinks, softcap, (const bf16_t*)gate, ldg);                                                                          \
+                       single_below, sinks, softcap, (const bf16_t*)gate, ldg, keep_first, score_bias);                                                                          \
   }
   // Two wave groups halve the walk of a tile over its keys; one group leaves LDS for a second
   // workgroup on the compute unit.  The first serves a step with few tiles, the second one with many.

@@ -48,6 +48,82 @@ extern "C" int mgpt_rms_norm_store(const void* src, int dtype, long ld, const fl
   return mgpt_last_error();
 }
 
+// A latent with a rotated part.  A cached row is [c: rank | kr: rot_dim | zeros up to row_width]: c as above,
+// kr one key part that all heads share, rotated by the token's position; a query head is [plain: head_dim |
+// rotated: rot_dim] and its rotated part is rotated in place.  Rotation of pairs (i, i + rot_dim / 2) by the angle
+// position * freq[i], cosine and sine both times rot_mag, in 32-bit.  One workgroup a token.  Without a pool
+// (a layer that reads another layer's latents) only the queries are rotated.
+#define LP_MAX_HALF 256
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prepare_kernel(
+    T* __restrict__ z, long ldz, int q_off, int n_head, int head_dim, int rot_dim, int c_off, int rank,
+    const float* __restrict__ gain, float eps, const int* __restrict__ positions, const float* __restrict__ freq,
+    float rot_mag, T* __restrict__ pool, int row_width, const int* __restrict__ slot_mapping, int n_tokens) {
+  __shared__ float cos_s[LP_MAX_HALF], sin_s[LP_MAX_HALF];
+  __shared__ float red_s[4];
+  const int n = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = rot_dim / 2;
+  const float p = (float)positions[n];
+  for (int i = tid; i < half; i += 256) {
+    const float a = p * freq[i];
+    cos_s[i] = cosf(a) * rot_mag;
+    sin_s[i] = sinf(a) * rot_mag;
+  }
+  T* row = z + (long)n * ldz;
+  const int slot = pool ? slot_mapping[n] : -1;
+  float ss = 0.f;
+  if (slot >= 0)
+    for (int c = tid; c < rank; c += 256) {
+      const float v = to_float<T>(row[c_off + c]);
+      ss = fmaf(v, v, ss);
+    }
+  ss = wave_sum(ss);
+  if (lane == 0) red_s[wave] = ss;
+  __syncthreads();
+  for (int idx = tid; idx < n_head * half; idx += 256) {
+    const int h = idx / half, i = idx - h * half;
+    T* at = row + q_off + (long)h * (head_dim + rot_dim) + head_dim;
+    const float u = to_float<T>(at[i]), w = to_float<T>(at[i + half]);
+    at[i] = from_float<T>(u * cos_s[i] - w * sin_s[i]);
+    at[i + half] = from_float<T>(w * cos_s[i] + u * sin_s[i]);
+  }
+  if (slot < 0) return;
+  const float inv = 1.0f / sqrtf(((red_s[0] + red_s[1]) + (red_s[2] + red_s[3])) / (float)rank + eps);
+  T* dst = pool + (long)slot * row_width;
+  for (int c = tid; c < rank; c += 256) dst[c] = from_float<T>(to_float<T>(row[c_off + c]) * inv * gain[c]);
+  for (int i = tid; i < half; i += 256) {
+    const float u = to_float<T>(row[c_off + rank + i]), w = to_float<T>(row[c_off + rank + i + half]);
+    dst[rank + i] = from_float<T>(u * cos_s[i] - w * sin_s[i]);
+    dst[rank + i + half] = from_float<T>(w * cos_s[i] + u * sin_s[i]);
+  }
+  for (int c = rank + rot_dim + tid; c < row_width; c += 256) dst[c] = from_float<T>(0.f);
+}
+
+// z: the step's projected rows (queries at q_off, n_head heads of head_dim + rot_dim; the latent's rank + rot_dim
+// columns at c_off); pool: the latent pages with rows of row_width >= rank + rot_dim values, or null.
+extern "C" int mgpt_latent_prepare(void* z, int dtype, long ldz, int q_off, int n_head, int head_dim, int rot_dim,
+                                   int c_off, int rank, const float* gain, float eps, const int* positions,
+                                   const float* freq, float rot_mag, void* pool, int row_width,
+                                   const int* slot_mapping, int n_tokens, hipStream_t stream) {
+  if (n_tokens == 0) return MGPT_OK;
+  if (!z || !positions || !freq || (pool && (!gain || !slot_mapping))) return MGPT_ERR_NULL;
+  if (n_tokens < 0 || n_head <= 0 || head_dim < 0 || rot_dim <= 0 || (rot_dim & 1) || rot_dim / 2 > LP_MAX_HALF ||
+      q_off < 0 || ldz < q_off + (long)n_head * (head_dim + rot_dim) ||
+      (pool && (rank <= 0 || row_width < rank + rot_dim || c_off < 0 || ldz < c_off + rank + rot_dim)))
+    return MGPT_ERR_BAD_SHAPE;
+  if (dtype == MGPT_F32)
+    hipLaunchKernelGGL(latent_prepare_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, (float*)z, ldz, q_off, n_head,
+                       head_dim, rot_dim, c_off, rank, gain, eps, positions, freq, rot_mag, (float*)pool, row_width,
+                       slot_mapping, n_tokens);
+  else if (dtype == MGPT_BF16)
+    hipLaunchKernelGGL(latent_prepare_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, (bf16_t*)z, ldz, q_off, n_head,
+                       head_dim, rot_dim, c_off, rank, gain, eps, positions, freq, rot_mag, (bf16_t*)pool, row_width,
+                       slot_mapping, n_tokens);
+  else
+    return MGPT_ERR_BAD_DTYPE;
+  return mgpt_last_error();
+}
+
 // out[n][h][o] = sum_i a[n][h][i] * w[h][o][i], optionally times sigmoid(gate[n][h][o]).
 // A workgroup owns 16 rows x 16 columns of one head, one element a thread; k runs 0..K-1 in order
 // for every element, so a row's result does not depend on the other rows of the launch.

@@ -10,17 +10,20 @@ extern "C" {
 int mgpt_paged_attention_split_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const
     void* vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int*
     q_req, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
+    const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const float* score_bias,
+    hipStream_t stream);
 // attention_decode.hip
 int mgpt_paged_attention_split_fast_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool,
     const void* vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const
     int* q_req, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
+    const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const float* score_bias,
+    hipStream_t stream);
 // attention_decode_wide.hip
 int mgpt_paged_attention_decode_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const
     void* vpool, const int* block_tables, int max_blocks, const int* positions, const int* q_req, const int*
     cu_q, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, int num_pages, float scale,
-    int window, int identity, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
+    int window, int identity, const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const
+    float* score_bias, hipStream_t stream);
 // attention_generic.hip
 int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int v_off, void* kpool, void* vpool, const
     int* slot_mapping, int n_tokens, int n_kv_head, int head_dim, int page_size, hipStream_t stream);
@@ -28,12 +31,14 @@ int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int v_off, voi
 int mgpt_paged_attention_generic(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window, int dtype,
-    int fast_exp, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
+    int fast_exp, const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const float*
+    score_bias, hipStream_t stream);
 // attention_prefill.hip
 int mgpt_prefill_attention_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req, int
     max_q_len, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window, int
-    single_below, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
+    single_below, const float* sinks, float softcap, const void* gate, long ldg, int keep_first, const float*
+    score_bias, hipStream_t stream);
 // embed_norm.hip
 int mgpt_embed(const int* ids, const int* pos, const void* tok, const void* postab, float* x, int n_tokens,
     int width, int table_dtype, hipStream_t stream);
@@ -125,10 +130,24 @@ int mgpt_scale_softcap(float* logits, long ld, int n_rows, int vocab, float scal
 // latent.hip
 int mgpt_rms_norm_store(const void* src, int dtype, long ld, const float* gain, float eps, void* pool, const int*
     slot_mapping, int n_tokens, int rank, hipStream_t stream);
+int mgpt_latent_prepare(void* z, int dtype, long ldz, int q_off, int n_head, int head_dim, int rot_dim, int c_off,
+    int rank, const float* gain, float eps, const int* positions, const float* freq, float rot_mag, void* pool,
+    int row_width, const int* slot_mapping, int n_tokens, hipStream_t stream);
 int mgpt_heads_linear(const void* a, long lda, const void* w, void* out, long ldo, const void* gate, long ldg,
     int n_rows, int n_head, int n_out, int k_dim, int dtype, int fast, hipStream_t stream);
 int mgpt_heads_linear_mfma(const void* a, long lda, const void* w, void* out, long ldo, const void* gate, long ldg,
     int n_rows, int n_head, int n_out, int k_dim, hipStream_t stream);
+// token_shift.hip
+int mgpt_parallel_norm(float* x, float* y, float mult, const float* gain, float offset, float eps, void* h, void* hs,
+    int dtype, const float* shift, float* state, long ld_state, const int* state_slots, const int* q_req,
+    const int* positions, int n_rows, int width, hipStream_t stream);
+int mgpt_token_shift(const void* h, void* hs, int dtype, const float* shift, const float* state, long ld_state,
+    const int* state_slots, const int* q_req, const int* cu_q, const int* positions, int n_rows, int width,
+    hipStream_t stream);
+int mgpt_token_shift_keep(const void* h, int dtype, float* state, long ld_state, const int* state_slots,
+    const int* cu_q, int n_req, int width, hipStream_t stream);
+int mgpt_xielu(const void* z, long ldz, void* out, long ldo, int dtype, const float* coef, int n_rows, int hidden,
+    int fast, hipStream_t stream);
 // experts.hip
 int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int n_rows, int hidden, int dtype, int fast,
     int kind, hipStream_t stream);
@@ -176,7 +195,8 @@ int mgpt_short_conv(const void* u, int dtype, long ldu, int u_off, const float* 
 int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head, int n_kv_head,
     int head_dim, int value_dim, int head_stride, const int* positions, const float* freq, int rot_dims, float norm_eps,
     const float* mix_lambda, void* v_other, long ld_other, int mix_mode, void* kpool, void* vpool,
-    const int* slot_mapping, int page_size, int n_tokens, hipStream_t stream);
+    const int* slot_mapping, int page_size, int n_tokens, int norm_mode, const float* q_norm_w, const float* k_norm_w,
+    int v_from_k, float rot_mag, hipStream_t stream);
 // decay_state.hip
 int mgpt_decay_state(const void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int g_off, int n_head,
     int head_dim, int value_dim, int act, const int* positions, const float* freq, int rot_dims, float k_scale,
@@ -224,6 +244,11 @@ int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_st
   X(mgpt_streams_step) \
   X(mgpt_scale_softcap) \
   X(mgpt_rms_norm_store) \
+  X(mgpt_latent_prepare) \
+  X(mgpt_parallel_norm) \
+  X(mgpt_token_shift) \
+  X(mgpt_token_shift_keep) \
+  X(mgpt_xielu) \
   X(mgpt_heads_linear) \
   X(mgpt_heads_linear_mfma) \
   X(mgpt_grouped_linear_mfma) \

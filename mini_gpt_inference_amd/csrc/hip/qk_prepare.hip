@@ -6,8 +6,13 @@
 //    a = position * freq[i].  freq is a float32 table made by the host (so base, scaling and any
 //    other rule for the frequencies are the caller's); position, angle, sine and cosine are
 //    float32, with the full-range sine and cosine.  The other channels pass unchanged.
+//    With `rot_mag` every cosine and sine is multiplied by that number;
 //  - optionally each query and key head divided by its root mean square over its `head_dim` real
-//    channels (eps inside the root), after the rotation;
+//    channels (eps inside the root), after the rotation (norm_mode 0 with norm_eps >= 0);
+//  - or, before the rotation, an RMS norm with weights: head by head with one weight vector [head_dim] for all
+//    query heads and one for all key heads (norm_mode 1), or over all of a token's query channels at once (and
+//    all of its key channels) with weights [heads * head_dim] (norm_mode 2);
+//  - with `v_from_k` the values are the keys as projected (before norm and rotation), and z holds no values;
 //  - optionally values mixed with those that another layer made for the same token:
 //    v <- (1 - lambda) v + lambda v_other (mode 2), or kept for such layers (mode 1);
 //  - queries written back in place; keys and values stored into their page (slot_mapping).
@@ -25,9 +30,11 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     int head_dim, int value_dim, int head_stride, const int* __restrict__ positions, const float* __restrict__ freq, int rot_dims,
     float norm_eps, const float* __restrict__ mix_lambda, void* __restrict__ v_other, long ld_other, int mix_mode,
     void* __restrict__ kpool, void* __restrict__ vpool, const int* __restrict__ slot_mapping, int page_size,
-    int n_tokens) {
+    int n_tokens, int norm_mode, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, int v_from_k,
+    float rot_mag) {
   __shared__ float cos_s[QKP_MAX_DIM / 2], sin_s[QKP_MAX_DIM / 2];
   __shared__ float head_s[4][QKP_MAX_DIM];
+  __shared__ float red_s[8];
   const int n = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int half = rot_dims / 2;
@@ -35,16 +42,39 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const float p = (float)positions[n];
     for (int i = threadIdx.x; i < half; i += 256) {
       const float a = p * freq[i];
-      cos_s[i] = cosf(a);
-      sin_s[i] = sinf(a);
+      cos_s[i] = cosf(a) * rot_mag;
+      sin_s[i] = sinf(a) * rot_mag;
     }
+  }
+  const long row = (long)n * ldz;
+  float whole_q = 1.0f, whole_k = 1.0f;   // norm_mode 2: what all query (key) channels of the token are multiplied by
+  if (norm_mode == 2) {
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < n_head * head_dim; i += 256) {
+      const int hh = i / head_dim;
+      const float v = load_f(z, dtype, row + q_off + (long)hh * head_stride + (i - hh * head_dim));
+      sq = fmaf(v, v, sq);
+    }
+    for (int i = threadIdx.x; i < n_kv_head * head_dim; i += 256) {
+      const int hh = i / head_dim;
+      const float v = load_f(z, dtype, row + k_off + (long)hh * head_stride + (i - hh * head_dim));
+      sk = fmaf(v, v, sk);
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if (lane == 0) {
+      red_s[wave] = sq;
+      red_s[4 + wave] = sk;
+    }
+    __syncthreads();
+    whole_q = 1.0f / sqrtf(((red_s[0] + red_s[1]) + (red_s[2] + red_s[3])) / (float)(n_head * head_dim) + norm_eps);
+    whole_k = 1.0f / sqrtf(((red_s[4] + red_s[5]) + (red_s[6] + red_s[7])) / (float)(n_kv_head * head_dim) + norm_eps);
   }
   __syncthreads();
   const int slot = slot_mapping ? slot_mapping[n] : -1;
   const long page = slot >= 0 ? slot / page_size : 0;
   const int off = slot >= 0 ? slot - (int)page * page_size : 0;
   float* s = head_s[wave];
-  const long row = (long)n * ldz;
   for (int hh = wave; hh < n_head + n_kv_head; hh += 4) {
     const bool is_q = hh < n_head;
     const int g = is_q ? hh : hh - n_head;
@@ -52,6 +82,22 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     const long src = row + (is_q ? q_off : k_off) + (long)g * head_stride;
     for (int c = lane; c < head_dim; c += 64) s[c] = load_f(z, dtype, src + c);
     __builtin_amdgcn_wave_barrier();
+    const long dst = ((page * n_kv_head + g) * page_size + off) * (long)head_stride;
+    if (v_from_k && !is_q && slot >= 0)   // the values are the keys as projected
+      for (int c = lane; c < head_stride; c += 64) store_f(vpool, dtype, dst + c, c < head_dim ? s[c] : 0.f);
+    if (norm_mode == 1) {
+      float ss = 0.f;
+      for (int c = lane; c < head_dim; c += 64) ss = fmaf(s[c], s[c], ss);
+      const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)head_dim + norm_eps);
+      const float* w = is_q ? q_norm_w : k_norm_w;
+      for (int c = lane; c < head_dim; c += 64) s[c] = s[c] * inv * w[c];
+      __builtin_amdgcn_wave_barrier();
+    } else if (norm_mode == 2) {
+      const float inv = is_q ? whole_q : whole_k;
+      const float* w = (is_q ? q_norm_w : k_norm_w) + (long)g * head_dim;
+      for (int c = lane; c < head_dim; c += 64) s[c] = s[c] * inv * w[c];
+      __builtin_amdgcn_wave_barrier();
+    }
     if (freq) {
       for (int i = lane; i < half; i += 64) {
         const float u = s[i], w = s[i + half], co = cos_s[i], si = sin_s[i];
@@ -61,7 +107,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
       __builtin_amdgcn_wave_barrier();
     }
     float r = 1.0f;
-    if (norm_eps >= 0.f) {
+    if (norm_mode == 0 && norm_eps >= 0.f) {
       float ss = 0.f;
       for (int c = lane; c < head_dim; c += 64) ss = fmaf(s[c], s[c], ss);
       r = 1.0f / sqrtf(wave_sum(ss) / (float)head_dim + norm_eps);
@@ -69,8 +115,11 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     if (is_q) {
       for (int c = lane; c < head_dim; c += 64) store_f(z, dtype, src + c, s[c] * r);
     } else if (slot >= 0) {
-      const long dst = ((page * n_kv_head + g) * page_size + off) * (long)head_stride;
       for (int c = lane; c < head_stride; c += 64) store_f(kpool, dtype, dst + c, c < head_dim ? s[c] * r : 0.f);
+      if (v_from_k) {
+        __builtin_amdgcn_wave_barrier();
+        continue;
+      }
       const long vsrc = row + v_off + (long)g * head_stride;
       const long osrc = (long)n * ld_other + (long)g * value_dim;
       const float lam = mix_mode == 2 ? mix_lambda[0] : 0.f;
@@ -94,6 +143,7 @@ extern "C" int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_of
                                int head_dim, int value_dim, int head_stride, const int* positions, const float* freq, int rot_dims,
                                float norm_eps, const float* mix_lambda, void* v_other, long ld_other, int mix_mode,
                                void* kpool, void* vpool, const int* slot_mapping, int page_size, int n_tokens,
+                               int norm_mode, const float* q_norm_w, const float* k_norm_w, int v_from_k, float rot_mag,
                                hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!z || (freq && !positions) || (kpool && (!vpool || !slot_mapping))) return MGPT_ERR_NULL;
@@ -102,8 +152,12 @@ extern "C" int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_of
       rot_dims < 0 || (rot_dims & 1) || rot_dims > head_dim || (kpool && page_size <= 0) || mix_mode < 0 || mix_mode > 2)
     return MGPT_ERR_BAD_SHAPE;
   if (mix_mode && (!v_other || (mix_mode == 2 && !mix_lambda))) return MGPT_ERR_NULL;
+  if (norm_mode < 0 || norm_mode > 2 || (norm_mode && !(norm_eps >= 0.f)) || (v_from_k && (mix_mode || value_dim != head_dim)))
+    return MGPT_ERR_BAD_SHAPE;
+  if (norm_mode && (!q_norm_w || !k_norm_w)) return MGPT_ERR_NULL;
   hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(256), 0, stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
                      n_kv_head, head_dim, value_dim, head_stride, positions, rot_dims ? freq : nullptr, rot_dims, norm_eps, mix_lambda,
-                     v_other, ld_other, mix_mode, kpool, vpool, slot_mapping, page_size, n_tokens);
+                     v_other, ld_other, mix_mode, kpool, vpool, slot_mapping, page_size, n_tokens, norm_mode, q_norm_w, k_norm_w,
+                     v_from_k, rot_mag);
   return mgpt_last_error();
 }

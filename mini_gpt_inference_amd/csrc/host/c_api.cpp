@@ -31,10 +31,10 @@ const char* mgpt_host_last_error() { return g_last_error.c_str(); }
 
 // ---------------------------------------------------------------- cache manager
 void* mgpt_cache_create(int n_groups, const int* page_sizes, const int* num_pages, const int* windows,
-                        int max_requests) {
+                        const int* keep_firsts, int max_requests) {
   GUARD_BEGIN
   std::vector<GroupSpec> groups;
-  for (int g = 0; g < n_groups; ++g) groups.push_back({page_sizes[g], num_pages[g], windows[g]});
+  for (int g = 0; g < n_groups; ++g) groups.push_back({page_sizes[g], num_pages[g], windows[g], keep_firsts ? keep_firsts[g] : 0});
   return new CacheManager(groups, max_requests);
   GUARD_END(nullptr)
 }

@@ -9,8 +9,8 @@ CacheManager::CacheManager(const std::vector<GroupSpec>& groups, int max_request
   if (groups.empty()) throw std::invalid_argument("at least one cache group is needed");
   if (max_requests <= 0) throw std::invalid_argument("max_requests must be positive");
   for (const GroupSpec& g : groups_) {
-    if (g.page_size <= 0 || g.num_pages <= 0 || g.window < 0)
-      throw std::invalid_argument("bad cache group: page_size and num_pages > 0, window >= 0");
+    if (g.page_size <= 0 || g.num_pages <= 0 || g.window < 0 || g.keep_first < 0)
+      throw std::invalid_argument("bad cache group: page_size and num_pages > 0, window and keep_first >= 0");
     // ids 0..n-1, taken from the end (src/minigpt_infer/cache/paged.py:39,63)
     std::vector<int> ids(g.num_pages);
     for (int i = 0; i < g.num_pages; ++i) ids[i] = i;
@@ -83,7 +83,9 @@ int CacheManager::release_passed(int slot, int n_computed) {
     const int earliest = n_computed - w + 1;
     if (earliest <= 0) continue;
     const int keep_from = std::min(earliest / groups_[g].page_size, (int)s.tables[g].size());
-    for (int p = s.first_live[g]; p < keep_from; ++p) {
+    // pages that hold one of the kept first positions stay
+    const int kept = (groups_[g].keep_first + groups_[g].page_size - 1) / groups_[g].page_size;
+    for (int p = std::max(s.first_live[g], kept); p < keep_from; ++p) {
       if (s.tables[g][p] >= 0) {
         free_pages_[g].push_back(s.tables[g][p]);
         s.tables[g][p] = -1;

@@ -17,6 +17,7 @@ struct GroupSpec {
   int page_size;  // tokens per page
   int num_pages;  // pages in this group's pool
   int window;     // 0: a query sees all earlier keys; w > 0: only the last w positions
+  int keep_first = 0;  // with a window: every query also sees the first keep_first positions, whose pages stay
 };
 
 class CacheManager {
@@ -40,7 +41,8 @@ class CacheManager {
   // group (pages a window has already released stay released).  All or nothing:
   // returns false and changes nothing when some group has too few free pages.
   bool reserve(int slot, int n_tokens);
-  // Give back the pages of window groups that no query at position >= n_computed can see.
+  // Give back the pages of window groups that no query at position >= n_computed can see (the pages of a
+  // group's kept first positions are never among them).
   // Returns the number of pages released.
   int release_passed(int slot, int n_computed);
   // Give back every page of the slot and the slot itself.  False if the slot is not live.

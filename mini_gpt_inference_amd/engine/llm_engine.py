@@ -173,7 +173,7 @@ class LLMEngine:
         pages = plan_group_pages(layout.groups, engine_config.block_size, engine_config.num_blocks,
                                  engine_config.kv_cache_bytes, 2 if self.dtype == torch.bfloat16 else 4,
                                  model.spec.max_positions)
-        geometry = [GroupGeometry(engine_config.block_size, n, g.window) for g, n in zip(layout.groups, pages)]
+        geometry = [GroupGeometry(engine_config.block_size, n, g.window, g.keep_first) for g, n in zip(layout.groups, pages)]
         self.cache = CacheManager(geometry, engine_config.max_batch_size)
         self.store = KVStore(layout, geometry, engine_config.max_batch_size, self.dtype, self.device)
         max_positions = model.spec.max_positions
@@ -432,7 +432,7 @@ class LLMEngine:
         computed = 0
         for sid in self.scheduler.running:
             n = self.scheduler.info(sid).num_computed
-            computed += min(n, geometry.window) if geometry.window else n
+            computed += min(n, geometry.window + geometry.keep_first) if geometry.window else n
         return {"free_blocks": free, "allocated_blocks": allocated,
                 "internal_fragmentation_slots": max(0, allocated * geometry.page_size - computed)}
 

@@ -15,7 +15,7 @@ from ..weights.loader import load_model
 from .step import ModelRunner
 
 PAGE_SIZE = 16   # tokens per cache page; divides the 64-token rounding of max_tokens
-MAX_LIVE = 8     # request slots
+MAX_LIVE = 4     # request slots
 
 
 class TraceError(RuntimeError):
@@ -33,7 +33,7 @@ class TraceReplayer:
         self.page_size = page_size
         self.num_pages = max(1, -(-int(max_tokens) // page_size))
         layout = self.model.cache_layout
-        geometry = [GroupGeometry(page_size, self.num_pages, g.window) for g in layout.groups]
+        geometry = [GroupGeometry(page_size, self.num_pages, g.window, g.keep_first) for g in layout.groups]
         self.cache = CacheManager(geometry, max_live)
         self.store = KVStore(layout, geometry, max_live, self.dtype, self.device, poison=poison)
         self.runner = ModelRunner(self.model, self.cache, self.store, self.dtype, self.device,

@@ -8,11 +8,12 @@ from . import kernels
 
 
 def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int, sinks=None,
-                softcap: float = 0.0, gate=None) -> bool:
+                softcap: float = 0.0, gate=None, keep_first: int = 0, score_bias=None) -> bool:
     """A step with prompt portions.  The requests that lead the step with one token each (a scheduler
     puts the decoding requests first) go to the decode kernel, token n being request n; the rest,
     prompt portions mostly, to the MFMA tile kernel, which would spend a 64-query tile on a single
     token.  False, having launched nothing, if the tile kernel does not take the case."""
+    mask = {"keep_first": keep_first, "score_bias": score_bias}
     q_lens = ctx.host_q_lens
     lead = 0
     if q_lens is not None:
@@ -21,64 +22,68 @@ def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, w
     rest = ctx.n_req - lead
     if lead and rest and kernels.prefill_attention_bf16(
             q, out, k_pool, v_pool, group.block_tables[lead:], ctx.cu_q[lead:], ctx.seq_lens[lead:], rest,
-            ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate):
+            ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate, **mask):
         if kernels.paged_attention_decode_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req,
                                                lead, n_head, scale, window, identity=True, sinks=sinks,
-                                               softcap=softcap, gate=gate):
+                                               softcap=softcap, gate=gate, **mask):
             return True
         # the decode kernel refuses this head or page size: the tile kernel for the leading requests too
         return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
-                                              lead, 1, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate)
+                                              lead, 1, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate, **mask)
     return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                           ctx.n_req, ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap,
-                                          gate=gate)
+                                          gate=gate, **mask)
 
 
 def _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int, sinks=None,
-                       softcap: float = 0.0, gate=None) -> bool:
+                       softcap: float = 0.0, gate=None, keep_first: int = 0, score_bias=None) -> bool:
     """A step with prompt portions that is padded to its bucket's sizes (a graph replays it for every
     step of the bucket): which request brings how many tokens is known on the device only.  The
     decode kernel goes over the step's first `ctx.lead_cap` tokens (decoding requests lead a step)
     and leaves out those of requests with several tokens; the tile kernel goes over all requests and
     leaves out those whose one token the decode kernel had; requests and tokens of the padding have
     neither.  False if the tile kernel refuses (the caller's general kernel then does all tokens again)."""
+    mask = {"keep_first": keep_first, "score_bias": score_bias}
     r = ctx.cu_q.numel() - 1
     lead = min(ctx.lead_cap, ctx.n_rows)
     singles = lead > 0 and kernels.paged_attention_decode_bf16(
         q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, lead, n_head, scale, window,
-        cu_q=ctx.cu_q, sinks=sinks, softcap=softcap, gate=gate)
+        cu_q=ctx.cu_q, sinks=sinks, softcap=softcap, gate=gate, **mask)
     return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens, r,
                                           ctx.n_rows, n_head, scale, window, single_below=lead if singles else 0,
-                                          sinks=sinks, softcap=softcap, gate=gate)
+                                          sinks=sinks, softcap=softcap, gate=gate, **mask)
 
 
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                     group, n_head: int, scale: float, window: int, sinks=None, softcap: float = 0.0,
-                    gate=None) -> None:
+                    gate=None, keep_first: int = 0, score_bias=None) -> None:
     """Attention of the step's tokens (rows of q) over their requests' pages.  softcap > 0: scores
     pass cap * tanh(score / cap) before the softmax.  gate ([tokens, >= heads], the queries' dtype): a head's
-    output is multiplied by sigmoid(gate[token][head]).
+    output is multiplied by sigmoid(gate[token][head]).  keep_first: behind a window a query also sees the keys
+    at positions below keep_first.  score_bias (float32 [heads]): no softmax; a visible key's weight is
+    sigmoid(score + score_bias[head]).
 
     On the bfloat16 path a decode-only step (token n is request n's one token) uses the kernel
     laid out for a decode step's latency, steps with prompt portions the MFMA tile kernel and the
     rest the kernel that splits a query's keys over four waves; the 32-bit path and every shape
     those refuse use the general kernel, whose order of sums depends only on a query's position."""
     n, r = ctx.n_rows, ctx.cu_q.numel() - 1
+    mask = {"keep_first": keep_first, "score_bias": score_bias}
     if q.dtype == torch.bfloat16 and not ctx.exact:
         if ctx.decode_only and kernels.paged_attention_decode_bf16(
                 q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, n, n_head, scale, window,
-                identity=True, sinks=sinks, softcap=softcap, gate=gate):
+                identity=True, sinks=sinks, softcap=softcap, gate=gate, **mask):
             return
         if not ctx.decode_only and not ctx.padded and _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head, scale,
-                                                                  window, sinks, softcap, gate):
+                                                                  window, sinks, softcap, gate, keep_first, score_bias):
             return
         if not ctx.decode_only and ctx.padded and _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head,
-                                                                     scale, window, sinks, softcap, gate):
+                                                                     scale, window, sinks, softcap, gate, keep_first, score_bias):
             return
         if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                               ctx.q_req, n, r, n_head, scale, window, sinks=sinks, softcap=softcap,
-                                              gate=gate):
+                                              gate=gate, **mask):
             return
     kernels.paged_attention_generic(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                     ctx.q_req, n, r, n_head, scale, window, fast_exp=not ctx.exact, sinks=sinks,
-                                    softcap=softcap, gate=gate)
+                                    softcap=softcap, gate=gate, **mask)

@@ -178,6 +178,18 @@ def kv_write(qkv: torch.Tensor, k_off: int, v_off: int, k_pool: torch.Tensor, v_
     _check(rc, "kv_write")
 
 
+def _mask_args(keep_first: int, score_bias: Optional[torch.Tensor], n_head: int, sinks, softcap: float):
+    """(first positions that a window keeps, pointer of the per-head number added to a score before its sigmoid):
+    the two optional arguments behind the gate's.  With score_bias the weights are sigmoids and not a softmax, so
+    sinks and a score cap do not go with it."""
+    _need(int(keep_first) >= 0, "keep_first must not be negative")
+    if score_bias is not None:
+        _need(score_bias.is_cuda and score_bias.dtype == torch.float32 and score_bias.is_contiguous()
+              and score_bias.numel() == n_head, "score_bias must be float32 [n_head] on the GPU")
+        _need(sinks is None and not softcap > 0.0, "sigmoid weights take neither sinks nor a score cap")
+    return int(keep_first), _ptr(score_bias)
+
+
 def _gate_args(gate: Optional[torch.Tensor], q: torch.Tensor, n_tokens: int, n_head: int):
     """(pointer, row stride) of the optional gate [tokens, >= heads] in q's dtype: a head's attention output is
     multiplied by sigmoid(gate[token][head])."""
@@ -212,10 +224,13 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
                             block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                             q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
                             window: int = 0, fast_exp: bool = False, sinks: Optional[torch.Tensor] = None,
-                            softcap: float = 0.0, gate: Optional[torch.Tensor] = None) -> None:
+                            softcap: float = 0.0, gate: Optional[torch.Tensor] = None, keep_first: int = 0,
+                            score_bias: Optional[torch.Tensor] = None) -> None:
     """Causal attention of the step's tokens over their requests' pages (any q_len, any dtype).
     sinks: float32 [n_head], one more term exp(sinks[h]) in every softmax denominator of head h.
-    softcap > 0: every score becomes softcap * tanh(score / softcap) before the softmax."""
+    softcap > 0: every score becomes softcap * tanh(score / softcap) before the softmax.
+    keep_first: behind a window a query also sees the keys at positions below it.  score_bias: float32 [n_head];
+    a visible key's weight is sigmoid(score + score_bias[h]), not normalised over the keys."""
     n_kv_head, page_size, head_dim = _check_attention_args(
         q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
     _need(head_dim <= 512, f"head size {head_dim} exceeds the kernel's limit of 512")
@@ -223,7 +238,8 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
     rc = library.kernels().mgpt_paged_attention_generic(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _ptr(sinks), float(softcap), *_gate_args(gate, q, n_tokens, n_head), _stream())
+        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _ptr(sinks), float(softcap), *_gate_args(gate, q, n_tokens, n_head),
+        *_mask_args(keep_first, score_bias, n_head, sinks, softcap), _stream())
     _check(rc, "paged_attention_generic")
 
 
@@ -498,7 +514,8 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
                                block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                                q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
                                window: int = 0, fast: bool = True, sinks: Optional[torch.Tensor] = None,
-                               softcap: float = 0.0, gate: Optional[torch.Tensor] = None) -> bool:
+                               softcap: float = 0.0, gate: Optional[torch.Tensor] = None, keep_first: int = 0,
+                               score_bias: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 attention with each (token, head)'s keys split over four waves.  False if refused.
     fast=False keeps to the variant that takes every head size."""
     if q.dtype != torch.bfloat16:
@@ -514,7 +531,8 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
     rc = fn(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _ptr(sinks), float(softcap), *_gate_args(gate, q, n_tokens, n_head), _stream())
+        page_size, float(scale), int(window), _ptr(sinks), float(softcap), *_gate_args(gate, q, n_tokens, n_head),
+        *_mask_args(keep_first, score_bias, n_head, sinks, softcap), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_split_bf16")
@@ -526,7 +544,8 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
                                 n_tokens: int, n_head: int, scale: float, window: int = 0,
                                 identity: bool = False, cu_q: Optional[torch.Tensor] = None,
                                 sinks: Optional[torch.Tensor] = None, softcap: float = 0.0,
-                                gate: Optional[torch.Tensor] = None) -> bool:
+                                gate: Optional[torch.Tensor] = None, keep_first: int = 0,
+                                score_bias: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 attention for single tokens (one query per request and step), keys split over eight
     waves.  positions[n] is token n's absolute position, q_req[n] its block table row or -1 for a
     padded token; identity=True promises q_req[n] in (n, -1).  With cu_q (the requests' token offsets;
@@ -562,7 +581,7 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(positions), _ptr(q_req), _ptr(cu_q), n_tokens, n_head, n_kv_head, head_dim, page_size,
         num_pages, float(scale), int(window), 1 if identity else 0, _ptr(sinks), float(softcap),
-        *_gate_args(gate, q, n_tokens, n_head), _stream())
+        *_gate_args(gate, q, n_tokens, n_head), *_mask_args(keep_first, score_bias, n_head, sinks, softcap), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_decode_bf16")
@@ -673,7 +692,8 @@ def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Ten
                            block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, n_req: int,
                            max_q_len: int, n_head: int, scale: float, window: int = 0,
                            single_below: int = 0, sinks: Optional[torch.Tensor] = None, softcap: float = 0.0,
-                           gate: Optional[torch.Tensor] = None) -> bool:
+                           gate: Optional[torch.Tensor] = None, keep_first: int = 0,
+                           score_bias: Optional[torch.Tensor] = None) -> bool:
     """MFMA tile attention for steps with prompt portions (every request's tokens are consecutive
     rows of q from cu_q; a request may bring none).  Requests that bring exactly one token, and that
     among the step's first `single_below` tokens, are left to another kernel.  False when it does
@@ -701,7 +721,7 @@ def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Ten
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), n_req, max_q_len, n_head, n_kv_head, head_dim,
         page_size, float(scale), int(window), int(single_below), _ptr(sinks), float(softcap),
-        *_gate_args(gate, q, q.shape[0], n_head), _stream())
+        *_gate_args(gate, q, q.shape[0], n_head), *_mask_args(keep_first, score_bias, n_head, sinks, softcap), _stream())
     if rc == -2:
         return False
     _check(rc, "prefill_attention_bf16")
@@ -1064,6 +1084,113 @@ def rms_norm_store(src: torch.Tensor, gain: torch.Tensor, eps: float, pool: torc
     _check(rc, "rms_norm_store")
 
 
+def latent_prepare(z: torch.Tensor, q_off: int, n_head: int, head_dim: int, rot_dim: int, positions: torch.Tensor,
+                   freq: torch.Tensor, n_tokens: int, rot_magnitude: float = 1.0, c_off: int = 0, rank: int = 0,
+                   gain: Optional[torch.Tensor] = None, eps: float = 0.0, pool: Optional[torch.Tensor] = None,
+                   slot_mapping: Optional[torch.Tensor] = None) -> None:
+    """Latent attention with a rotated part: the last rot_dim channels of every query head (heads of head_dim +
+    rot_dim channels at q_off of z's rows) are rotated in place by the token's position; with `pool` (latent pages
+    whose rows hold at least rank + rot_dim values) the token's row becomes [rms_norm(z[c_off : c_off + rank]) * gain |
+    the next rot_dim columns of z, rotated | zeros].  freq: float32 [rot_dim / 2]."""
+    _need_cuda(z, positions, freq, gain, pool, slot_mapping)
+    _rows_2d("latent_prepare z", z, n_tokens)
+    _need(freq.dtype == torch.float32 and freq.is_contiguous() and freq.numel() * 2 == rot_dim, "latent_prepare: float32 frequencies [rot_dim / 2]")
+    _need_i32("positions", positions, n_tokens)
+    _need(z.shape[1] >= q_off + n_head * (head_dim + rot_dim), "latent_prepare: z is too narrow for the queries")
+    row_width = 0
+    if pool is not None:
+        _need(pool.dtype == z.dtype and pool.is_contiguous() and pool.dim() == 4 and pool.shape[1] == 1
+              and pool.shape[3] >= rank + rot_dim, "latent_prepare: the pool must be [pages, 1, page, >= rank + rot_dim] in z's dtype")
+        _need(gain is not None and gain.dtype == torch.float32 and gain.is_contiguous() and gain.numel() == rank,
+              "latent_prepare: gain must be float32 [rank]")
+        _need(z.shape[1] >= c_off + rank + rot_dim, "latent_prepare: z is too narrow for the latent")
+        _need_i32("slot_mapping", slot_mapping, n_tokens)
+        row_width = pool.shape[3]
+    rc = library.kernels().mgpt_latent_prepare(
+        _ptr(z), _dtype_code(z), z.stride(0), int(q_off), n_head, head_dim, rot_dim, int(c_off), int(rank), _ptr(gain),
+        float(eps), _ptr(positions), _ptr(freq), float(rot_magnitude), _ptr(pool), row_width, _ptr(slot_mapping), n_tokens,
+        _stream())
+    _check(rc, "latent_prepare")
+
+
+def parallel_norm(x: torch.Tensor, y: Optional[torch.Tensor], mult: float, n_rows: int, gain: Optional[torch.Tensor] = None,
+                  offset: float = 0.0, eps: float = 0.0, h: Optional[torch.Tensor] = None, hs: Optional[torch.Tensor] = None,
+                  shift: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
+                  state_slots: Optional[torch.Tensor] = None, q_req: Optional[torch.Tensor] = None,
+                  positions: Optional[torch.Tensor] = None) -> None:
+    """x += mult * y and y = 0 (y float32 rows like x, or None); with h: h = x / sqrt(mean(x^2) + eps) * (offset + gain);
+    with hs (only in a step whose requests bring one token each): hs = h + (kept - h) * shift with `kept` the
+    request's row of `state` (zeros at position 0), which then takes h."""
+    _need_cuda(x, y, gain, h, hs, shift, state, state_slots, q_req, positions)
+    width = x.shape[1]
+    for t in (x, y):
+        _need(t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.shape[1] == width and t.shape[0] >= n_rows),
+              "parallel_norm: x and y must be dense float32 rows of one width")
+    dtype = 0
+    if h is not None:
+        _need(gain is not None and gain.dtype == torch.float32 and gain.is_contiguous() and gain.numel() == width,
+              "parallel_norm: gain must be float32 [width]")
+        for t in (h, hs):
+            _need(t is None or (t.is_contiguous() and t.shape[1] == width and t.shape[0] >= n_rows and t.dtype == h.dtype),
+                  "parallel_norm: h and hs must be dense rows as wide as x, of one dtype")
+        dtype = _dtype_code(h)
+    ld_state = 0
+    if hs is not None:
+        _need(h is not None, "parallel_norm: the shift reads h")
+        ld_state = _need_shift_state(shift, state, state_slots, width)
+        _need_i32("q_req", q_req, n_rows)
+        _need_i32("positions", positions, n_rows)
+    rc = library.kernels().mgpt_parallel_norm(
+        _ptr(x), _ptr(y), float(mult), _ptr(gain), float(offset), float(eps), _ptr(h), _ptr(hs), dtype, _ptr(shift),
+        _ptr(state), ld_state, _ptr(state_slots), _ptr(q_req), _ptr(positions), n_rows, width, _stream())
+    _check(rc, "parallel_norm")
+
+
+def _need_shift_state(shift, state, state_slots, width: int) -> int:
+    _need(shift is not None and shift.dtype == torch.float32 and shift.is_contiguous() and shift.numel() == width,
+          "token shift: shift must be float32 [width]")
+    _need(state is not None and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= width, "token shift: the state pool must be float32 rows of at least the width")
+    _need(state_slots is not None and state_slots.dtype == torch.int32 and state_slots.is_contiguous(),
+          "token shift: state_slots must be int32")
+    return state.stride(0)
+
+
+def token_shift(h: torch.Tensor, hs: torch.Tensor, shift: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
+                q_req: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor, n_rows: int, n_req: int) -> None:
+    """hs = h + (h_before - h) * shift for every token of the step, h_before being the row before (same request),
+    the request's row of `state` for its first token of the step, zeros at position 0; then every request's row
+    of `state` takes the h of its last token."""
+    _need_cuda(h, hs, shift, state, state_slots, q_req, cu_q, positions)
+    width = h.shape[1]
+    _need(h.is_contiguous() and hs.is_contiguous() and hs.shape[1] == width and h.dtype == hs.dtype and h.shape[0] >= n_rows
+          and hs.shape[0] >= n_rows, "token_shift: h and hs must be dense rows of one width and dtype")
+    ld_state = _need_shift_state(shift, state, state_slots, width)
+    _need_i32("q_req", q_req, n_rows)
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need_i32("positions", positions, n_rows)
+    _need(state_slots.numel() >= n_req, "token_shift: a state slot per request")
+    lib = library.kernels()
+    rc = lib.mgpt_token_shift(_ptr(h), _ptr(hs), _dtype_code(h), _ptr(shift), _ptr(state), ld_state, _ptr(state_slots),
+                              _ptr(q_req), _ptr(cu_q), _ptr(positions), n_rows, width, _stream())
+    _check(rc, "token_shift")
+    rc = lib.mgpt_token_shift_keep(_ptr(h), _dtype_code(h), _ptr(state), ld_state, _ptr(state_slots), _ptr(cu_q), n_req,
+                                   width, _stream())
+    _check(rc, "token_shift_keep")
+
+
+def xielu(z: torch.Tensor, out: torch.Tensor, coef: torch.Tensor, n_rows: int, hidden: int, fast: bool = False) -> None:
+    """out = coef[0] z^2 + z / 2 where z > 0, coef[1] (exp(z) - 1 - z) + z / 2 elsewhere; coef float32 [2]."""
+    _need_cuda(z, out, coef)
+    _rows_2d("xielu z", z, n_rows)
+    _rows_2d("xielu out", out, n_rows)
+    _need(z.dtype == out.dtype and z.shape[1] >= hidden and out.shape[1] >= hidden, "xielu: rows of one dtype, at least `hidden` wide")
+    _need(coef.dtype == torch.float32 and coef.is_contiguous() and coef.numel() == 2, "xielu: coef must be float32 [2]")
+    rc = library.kernels().mgpt_xielu(_ptr(z), z.stride(0), _ptr(out), out.stride(0), _dtype_code(z), _ptr(coef), n_rows,
+                                      hidden, int(fast), _stream())
+    _check(rc, "xielu")
+
+
 def heads_linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_rows: int,
                  gate: Optional[torch.Tensor] = None, fast: bool = False) -> None:
     """out[n][h] = a[n][h] @ w[h].T for every head h, optionally times sigmoid(gate[n][h]).
@@ -1377,18 +1504,34 @@ def rms_post_norm(branches, x: torch.Tensor, gain_post: torch.Tensor, n_rows: in
     _check(rc, "rms_post_norm")
 
 
+QK_NORMS = {None: 0, "head": 1, "whole": 2}
+
+
 def qk_prepare(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int, n_kv_head: int, head_dim: int,
                value_dim: int, head_stride: int, n_tokens: int, positions: Optional[torch.Tensor] = None,
                freq: Optional[torch.Tensor] = None, norm_eps: Optional[float] = None,
                mix_lambda: Optional[torch.Tensor] = None, v_other: Optional[torch.Tensor] = None, mix_mode: int = 0,
                k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,
-               slot_mapping: Optional[torch.Tensor] = None) -> None:
+               slot_mapping: Optional[torch.Tensor] = None, norm: Optional[str] = None,
+               q_norm_weight: Optional[torch.Tensor] = None, k_norm_weight: Optional[torch.Tensor] = None,
+               values_from_keys: bool = False, rot_magnitude: float = 1.0) -> None:
     """Projected queries, keys and values of a step's tokens (rows of z; q heads at q_off, k heads at k_off, v heads
     at v_off, head_stride channels apart) made ready for attention: q and k rotated by position with the float32
     frequencies `freq` [rot_dims / 2] (pairs (i, i + rot_dims / 2)), then divided by their root mean square over
     head_dim channels if norm_eps is given; v kept for other layers in v_other (heads value_dim apart; mix_mode 1) or mixed with what
-    lies there, (1 - lambda) v + lambda v_other (mix_mode 2); q back in place, k and v into their pages."""
-    _need_cuda(z, positions, freq, mix_lambda, v_other, k_pool, v_pool, slot_mapping)
+    lies there, (1 - lambda) v + lambda v_other (mix_mode 2); q back in place, k and v into their pages.
+    norm "head" / "whole" (with norm_eps and float32 weights [head_dim] / [heads * head_dim] for q and for k): an RMS
+    norm with weights *before* the rotation, head by head with the heads sharing a weight vector, or over all of a
+    token's query (key) channels at once.  values_from_keys: the values are the keys as projected, z holds none.
+    rot_magnitude multiplies every cosine and sine."""
+    _need_cuda(z, positions, freq, mix_lambda, v_other, k_pool, v_pool, slot_mapping, q_norm_weight, k_norm_weight)
+    _need(norm in QK_NORMS, f"qk_prepare: norm {norm!r} is none of {sorted(QK_NORMS, key=str)}")
+    if norm is not None:
+        for w, heads in ((q_norm_weight, n_head), (k_norm_weight, n_kv_head)):
+            _need(norm_eps is not None and w is not None and w.dtype == torch.float32 and w.is_contiguous()
+                  and w.numel() == (head_dim if norm == "head" else heads * head_dim),
+                  "qk_prepare: a norm with weights needs eps and float32 weights of the head's (or the projection's) size")
+    _need(not values_from_keys or (value_dim == head_dim and mix_mode == 0), "qk_prepare: values that are the keys have their size")
     _rows_2d("qk_prepare z", z, n_tokens)
     rot_dims = 0
     if freq is not None:
@@ -1397,7 +1540,8 @@ def qk_prepare(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int,
         rot_dims = 2 * freq.numel()
     kv_span = (n_kv_head - 1) * head_stride
     _need(z.shape[1] >= max(q_off + (n_head - 1) * head_stride + head_dim, k_off + kv_span + head_dim,
-                            v_off + kv_span + head_stride if k_pool is not None else 0), "qk_prepare: z is too narrow")
+                            v_off + kv_span + head_stride if k_pool is not None and not values_from_keys else 0),
+          "qk_prepare: z is too narrow")
     page_size = 0
     if k_pool is not None:
         _need(v_pool is not None and k_pool.dtype == z.dtype and v_pool.dtype == z.dtype and k_pool.dim() == 4
@@ -1416,7 +1560,8 @@ def qk_prepare(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int,
         _ptr(z), _dtype_code(z), z.stride(0), q_off, k_off, v_off, n_head, n_kv_head, head_dim, value_dim, head_stride,
         _ptr(positions), _ptr(freq), rot_dims, -1.0 if norm_eps is None else float(norm_eps), _ptr(mix_lambda),
         _ptr(v_other), v_other.stride(0) if v_other is not None else 0, int(mix_mode), _ptr(k_pool), _ptr(v_pool),
-        _ptr(slot_mapping), page_size, n_tokens, _stream())
+        _ptr(slot_mapping), page_size, n_tokens, QK_NORMS[norm], _ptr(q_norm_weight) if norm else None,
+        _ptr(k_norm_weight) if norm else None, int(values_from_keys), float(rot_magnitude), _stream())
     _check(rc, "qk_prepare")
 
 

@@ -39,7 +39,7 @@ def kernels() -> ctypes.CDLL:
         lib.mgpt_layernorm.argtypes = [P, P, P, P, P, I, I, F, I, P]
         lib.mgpt_linear_generic.argtypes = [P, I, L, P, I, P, P, I, L, I, I, I, I, P]
         lib.mgpt_kv_write.argtypes = [P, I, L, I, I, P, P, P, I, I, I, I, P]
-        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, F, P, L, P]
+        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, F, P, L, I, P, P]
         lib.mgpt_sample.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P, P, P, I, P]
         lib.mgpt_sample_advance.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P,
                                             P, P, P, P, P, P, P, I, I, I, I, P, P, I, I, P, P, I, P]
@@ -127,15 +127,15 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_linear_skinny_partials": [I, I, I, I, I],
         "mgpt_linear_skinny_row_groups": [I, I, I],
         "mgpt_fold_layernorm": [P, P, P, P, P, P, P, I, I, P],
-        "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P, L, P],
-        "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P, L, P],
-        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P, F, P, L, P],
+        "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P, L, I, P, P],
+        "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P, L, I, P, P],
+        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P, F, P, L, I, P, P],
         "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_shape": [I, I, P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_partials": [I, I, I, I],
         "mgpt_linear_mfma_parts": [P, L, P, P, P, L, I, I, I, P],
         "mgpt_linear_mfma_qkv": [P, L, P, P, P, L, I, I, I, P, P, P, I, I, I, I, I, I, P],
-        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, F, P, L, P],
+        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, F, P, L, I, P, P],
         # a residual that is still a sum: base, partials, n_parts, part_stride, token table, position table, ids, positions
         "mgpt_fused_attention_decode": [P, P, I, L, P, P, P, P, P, P, P, P, F, P, P, P, P, P, L, P, P, P, P, I, P, P,
                                         I, I, I, I, I, I, F, P],
@@ -156,13 +156,19 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         # latent attention
         "mgpt_rms_norm_store": [P, I, L, P, F, P, P, I, I, P],
         "mgpt_heads_linear": [P, L, P, P, L, P, L, I, I, I, I, I, I, P],
+        "mgpt_latent_prepare": [P, I, L, I, I, I, I, I, I, P, F, P, P, F, P, I, P, I, P],
+        # a layer whose sublayers read one norm, the mixer through a token shift; the xIELU activation
+        "mgpt_parallel_norm": [P, P, F, P, F, F, P, P, I, P, P, L, P, P, P, I, I, P],
+        "mgpt_token_shift": [P, P, I, P, P, L, P, P, P, P, I, I, P],
+        "mgpt_token_shift_keep": [P, I, P, L, P, P, I, I, P],
+        "mgpt_xielu": [P, L, P, L, I, P, I, I, I, P],
         "mgpt_heads_linear_mfma": [P, L, P, P, L, P, L, I, I, I, I, P],
         # gated feed-forwards and experts
         "mgpt_gated_unit": [P, L, P, L, I, I, I, I, I, P],
         # root-mean-square norms, rotation and the rest in front of attention, decaying state
         "mgpt_rms_norm": [P, I, L, P, P, F, F, F, P, I, L, I, P, I, L, I, P, L, I, I, I, I, I, I, P],
         "mgpt_rms_post_norm": [P, P, P, P, P, P, P, P, I, F, I, P, P, P, F, F, F, P, P, I, I, I, P],
-        "mgpt_qk_prepare": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, L, I, P, P, P, I, I, P],
+        "mgpt_qk_prepare": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, L, I, P, P, P, I, I, I, P, P, I, F, P],
         "mgpt_decay_state": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, F, P, I, L, P],
         "mgpt_decay_state_chunked": [P, I, L, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, I, P, P, L, P],
         "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, P, I, I, I, P],
@@ -194,7 +200,7 @@ def host() -> ctypes.CDLL:
         IP = POINTER(c_int)
         lib.mgpt_host_last_error.restype = c_char_p
         lib.mgpt_cache_create.restype = P
-        lib.mgpt_cache_create.argtypes = [I, IP, IP, IP, I]
+        lib.mgpt_cache_create.argtypes = [I, IP, IP, IP, IP, I]
         lib.mgpt_cache_destroy.argtypes = [P]
         lib.mgpt_cache_destroy.restype = None
         for name, args in {

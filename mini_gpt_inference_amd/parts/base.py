@@ -44,6 +44,7 @@ class KVNeed:
     head_dim: int
     window: int = 0   # 0: all earlier keys; w: the last w positions
     joint: bool = False   # keys and values are one tensor (a latent that both are made from): a page holds it once
+    keep_first: int = 0   # with a window: every query also sees the first keep_first positions of its request
     state_numel: int = 0  # float32 values per request that the mixer keeps beside its pages (the last inputs of a
                           # short convolution in front of its keys, say); 0: none
 

@@ -271,6 +271,89 @@ class SandwichNorm(Arrangement):
         ctx.pending_update = PendingSandwich([(ys[0], None)], x, parts["norm2b"], self.mult, n, True, self.scale2)
 
 
+@register_arrangement("parallel_shift")
+class ParallelShift(Arrangement):
+    """A layer with one norm whose sublayers all read it and are added together:
+
+        h = norm1(x);   x <- x + m * (mixer(shifted(h)) + ff(h))
+
+    with m = `residual_mult`; the feed-forward is optional.  With `token_shift` the mixer (not the feed-forward)
+    reads h blended with the previous token's: shifted(h)_t = h_t + (h_(t-1) - h_t) * shift, channel by channel,
+    `shift` a vector of the layer, h_(-1) = 0.  The h of a request's last token is kept per request in a
+    state pool of the arrangement's own.  norm1 is an RMS norm (kind "rms_norm") with a gain.
+
+    The sublayers are the framework's ordinary parts: they add their output into one cleared float32 buffer.
+    The addition to the residual is left pending and made by the next layer's norm kernel (or by whoever
+    reads the residual next)."""
+
+    graph_safe = True
+    plan_safe = True
+    takes_pending_update = True
+
+    def __init__(self, width: int, residual_mult: float = 1.0, feed_forward: bool = True, token_shift: bool = False) -> None:
+        self.width, self.mult = int(width), float(residual_mult)
+        self.has_feed_forward, self.has_shift = bool(feed_forward), bool(token_shift)
+        self.roles = ("norm1", "mixer") + (("feed_forward",) if self.has_feed_forward else ())
+        self.shift = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        return {"shift": WeightRequest((self.width,), VECTOR)} if self.has_shift else {}
+
+    def state_numel(self) -> int:
+        """float32 values kept per request: the last token's normed row."""
+        return self.width if self.has_shift else 0
+
+    def run(self, ctx, x, parts, bindings, position) -> None:
+        norm1 = parts["norm1"]
+        if not (hasattr(norm1, "offset") and getattr(norm1, "has_weight", False) and norm1.width == self.width):
+            raise ValueError("a parallel layer takes an RMS norm with a gain as wide as the model")
+        n, ws = ctx.n_rows, ctx.workspace
+        made = ws.generation
+        y = ws.get("parallel_sums", n, self.width, torch.float32)
+        if ws.generation != made:
+            y.zero_()       # cleared when it is made, and by the kernel that takes the sums out of it ever after
+        h = ws.get("normed", n, self.width, ctx.dtype)
+        hs = ws.get("normed_shifted", n, self.width, ctx.dtype) if self.has_shift else None
+        left, ctx.pending_update = ctx.pending_update, None
+        y_before, mult_before = None, 0.0
+        if isinstance(left, PendingParallel) and left.goes_with(x, n):
+            y_before, mult_before = left.y, left.mult     # the layer before's addition and this layer's norm in one kernel
+        elif left is not None:
+            left.run(None, None)
+        state = ctx.state_pools[bindings[STATE_ROLE].index] if self.has_shift else None
+        # every request brings one token: a row's neighbour in time is its request's kept row, and the same kernel
+        # shifts and keeps; else the shift reads the step's rows and runs behind the norm
+        single = self.has_shift and ctx.decode_only
+        kernels.parallel_norm(x, y_before, mult_before, n, gain=norm1.weight, offset=norm1.offset, eps=norm1.eps, h=h,
+                              hs=hs if single else None, shift=self.shift, state=state, state_slots=ctx.state_slots,
+                              q_req=ctx.q_req, positions=ctx.positions)
+        if self.has_shift and not single:
+            kernels.token_shift(h, hs, self.shift, state, ctx.state_slots, ctx.q_req, ctx.cu_q, ctx.positions, n,
+                                ctx.cu_q.numel() - 1)
+        parts["mixer"].forward_add(ctx, hs if self.has_shift else h, y, bindings["mixer"], position)
+        if self.has_feed_forward:
+            parts["feed_forward"].forward_add(ctx, h, y)
+        ctx.pending_update = PendingParallel(x, y, self.mult, n)
+
+
+STATE_ROLE = "arrangement"     # the name under which a run's bindings hold an arrangement's own state pool
+
+
+class PendingParallel:
+    """The sum of a parallel layer's sublayers that is still to be added to the residual: x += mult * y, y = 0."""
+
+    def __init__(self, x: torch.Tensor, y: torch.Tensor, mult: float, n_rows: int) -> None:
+        self.x, self.y, self.mult, self.n_rows = x, y, mult, n_rows
+
+    def goes_with(self, *args) -> bool:
+        """(x, n_rows): whether a parallel layer over these rows may make the addition in its norm kernel; asked
+        with anything else (another arrangement's norm), no."""
+        return len(args) == 2 and args[0] is self.x and args[1] == self.n_rows
+
+    def run(self, gain_next=None, h=None) -> None:
+        kernels.parallel_norm(self.x, self.y, self.mult, self.n_rows)
+
+
 class PendingSandwich:
     """A sublayer's output that is still to be normed and added to the residual: x += mult * norm(y).  Whoever
     reads x next makes the addition: a layer of the same kind together with its first norm (run(gain, h) also

@@ -10,7 +10,8 @@ from ..ops import kernels, residual
 from ..ops.linear import LazyNorm, as_tensor, linear, linear_add, packed_weight, plain_residual
 from .base import MATRIX, Part, StepContext, TABLE, VECTOR, WeightRequest, register_feed_forward
 
-_ACTIVATIONS = {"gelu_tanh": kernels.EPI_GELU}
+# activations of the dense feed-forward: an epilogue of the product kernels, or (None) a kernel of its own behind them
+_ACTIVATIONS = {"gelu_tanh": kernels.EPI_GELU, "xielu": None}
 
 
 class FeedForward(Part):
@@ -25,7 +26,8 @@ class FeedForward(Part):
 class DenseMLP(FeedForward):
     """u = h Wfc^T (+ b); g = 0.5 u (1 + tanh(sqrt(2/pi)(u + 0.044715 u^3))); m = g Wproj^T (+ b)
     (reference: src/minigpt_infer/model.py:96-101; there the hidden size is 4*n_embd, here it is
-    a parameter)."""
+    a parameter).  With activation "xielu" g is instead, from two stored numbers (p, q) (the tensor `act`),
+    softplus(p) u^2 + u / 2 for u > 0 and (1/2 + softplus(q)) (exp(u) - 1 - u) + u / 2 for u <= 0."""
 
     graph_safe = True
 
@@ -45,7 +47,17 @@ class DenseMLP(FeedForward):
         if self.has_bias:
             req["fc_bias"] = WeightRequest((self.hidden,), VECTOR)
             req["proj_bias"] = WeightRequest((self.width,), VECTOR)
+        if self.activation == "xielu":
+            req["act"] = WeightRequest((2,), VECTOR)
         return req
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        if self.activation == "xielu":
+            # the two branches' coefficients, made once: softplus(p) and 1/2 + softplus(q)
+            sp = torch.nn.functional.softplus(tensors["act"].to(torch.float32))
+            self.act_coef = torch.stack([sp[0], sp[1] + 0.5]).contiguous()
+        return None
 
     def _forward_add_fused(self, ctx: StepContext, h, x: torch.Tensor) -> bool:
         """A decode-only step of few rows: one kernel from the residual (a sum, as the kernels
@@ -78,7 +90,10 @@ class DenseMLP(FeedForward):
         plain_residual(ctx, h, x)
         n = ctx.n_rows
         u = ctx.workspace.get("ff_hidden", n, self.hidden, ctx.dtype)
-        linear(ctx, h, self.fc_weight, self.fc_bias, u, n, _ACTIVATIONS[self.activation])
+        epilogue = _ACTIVATIONS[self.activation]
+        linear(ctx, h, self.fc_weight, self.fc_bias, u, n, kernels.EPI_NONE if epilogue is None else epilogue)
+        if self.activation == "xielu":
+            kernels.xielu(u, u, self.act_coef, n, self.hidden, fast=not ctx.exact)
         # (a caller that hands over a LazyNorm of x itself knows that x may be left as a sum)
         linear_add(ctx, u, self.proj_weight, self.proj_bias, x, n,
                    may_leave_parts=isinstance(h, LazyNorm) and h.x is x)

@@ -141,18 +141,25 @@ class PagedCausalAttention(Mixer):
 @register_mixer("latent_attention")
 class LatentAttention(Mixer):
     """Attention whose keys and values are made from one small latent per token, which is all the
-    cache keeps (one joint tensor per page), without a position signal.
+    cache keeps (one joint tensor per page).
 
     c = rms_norm(h Wdkv^T) * gain, [rank], stored into the pages.  Per head a: q_a = h Wq_a^T [D],
     k_a = Wuk_a c [D], v_a = Wuv_a c [E]; S = (q_a . k_a) * scale over the keys at positions
     p - window < j <= p (window 0: all j <= p); softmax in float32 with one more term exp(sink_a) in
     the denominator that has no value; y = concat_a(P v_a) * sigmoid(h Wg^T); out = y Wo^T, added
-    into the residual.
+    into the residual.  The gate is a number per channel of y (`gate` "channel", Wg [H * E, W]) or a
+    number per head ("head", Wg [H, W]).
+
+    With `rot_dim` = P > 0 a position signal rides beside the latent: a query head is [D plain | P rotated]
+    channels (Wq has H (D + P) rows), Wdkv has rank + P rows of which the last P, not normed, are one key part
+    kr that all heads share, and S = (q_plain . k_a + rot(q_rot) . rot(kr)) * scale with `rotary` (the mixer's
+    own rotation over P channels).  The cache then keeps [c | rot(kr)] per token.
 
     The kernels never make k_a and v_a: (q_a . Wuk_a c) = (Wuk_a^T q_a) . c, so the queries are
-    folded onto the latent basis (one product per head), attention runs with one key/value head of
-    size `rank` that every query head shares, and its output sum_j P_j c_j is unfolded by Wuv_a
-    afterwards.  A layer with makes_latent=False has no Wdkv: it reads the pages that another run
+    folded onto the latent basis (one product per head, which passes the rotated part through), attention
+    runs with one key/value head of the cached row's size that every query head shares, and its output
+    sum_j P_j c_j is unfolded by Wuv_a afterwards (which has no columns for the rotated part).  A layer with
+    makes_latent=False has no Wdkv: it reads the pages that another run
     of the same step wrote (LayerRun.reads_cache_of), with its own Wuk, Wuv, window and the rest."""
 
     graph_safe = True
@@ -163,49 +170,86 @@ class LatentAttention(Mixer):
     JOINT_PRODUCT_MAX_WORK = 4 << 20     # rows x (query + gate columns); a smaller product has no full round to lose
 
     def __init__(self, width: int, n_head: int, head_dim: int, value_dim: int, rank: int, scale: float,
-                 window: int = 0, eps: float = 1e-6, makes_latent: bool = True) -> None:
+                 window: int = 0, eps: float = 1e-6, makes_latent: bool = True, rot_dim: int = 0,
+                 rotary: Optional[dict] = None, gate: str = "channel") -> None:
         self.width, self.n_head, self.head_dim = int(width), int(n_head), int(head_dim)
         self.value_dim, self.rank = int(value_dim), int(rank)
         self.scale, self.window, self.eps = float(scale), int(window), float(eps)
         self.makes_latent = bool(makes_latent)
-        if not 0 < self.rank <= 512:
-            raise ValueError(f"latent size {self.rank}: the attention kernels take up to 512")
-        self.q_width, self.g_width = self.n_head * self.head_dim, self.n_head * self.value_dim
+        self.rot_dim = int(rot_dim or 0)
+        self.rotation = _own_rotation(rotary) if self.rot_dim else None
+        if self.rot_dim and (self.rotation is None or self.rotation.dims != self.rot_dim):
+            raise ValueError("a latent with a rotated part needs a rotation over exactly rot_dim channels")
+        if gate not in ("channel", "head"):
+            raise ValueError(f"gate {gate!r} is neither 'channel' nor 'head'")
+        self.head_gate = gate == "head"
+        # what a cached row holds: the latent alone, or the latent and the rotated key part (rows then
+        # start 16 bytes apart in bfloat16 too)
+        self.row = self.rank if not self.rot_dim else -(-(self.rank + self.rot_dim) // 8) * 8
+        if not 0 < self.row <= 512:
+            raise ValueError(f"latent size {self.row}: the attention kernels take up to 512")
+        self.q_head = self.head_dim + self.rot_dim
+        self.q_width = self.n_head * self.q_head
+        self.y_width = self.n_head * self.value_dim
+        self.g_width = self.n_head if self.head_gate else self.y_width
         self.in_weight = self.uk_folded = self.uv_heads = None
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
         req = {"q_weight": WeightRequest((self.q_width, self.width), MATRIX),
                "gate_weight": WeightRequest((self.g_width, self.width), MATRIX),
-               "uk_weight": WeightRequest((self.q_width, self.rank), MATRIX),
-               "uv_weight": WeightRequest((self.g_width, self.rank), MATRIX),
+               "uk_weight": WeightRequest((self.n_head * self.head_dim, self.rank), MATRIX),
+               "uv_weight": WeightRequest((self.y_width, self.rank), MATRIX),
                "sink": WeightRequest((self.n_head,), VECTOR),
-               "out_weight": WeightRequest((self.width, self.g_width), MATRIX)}
+               "out_weight": WeightRequest((self.width, self.y_width), MATRIX)}
         if self.makes_latent:
-            req["dkv_weight"] = WeightRequest((self.rank, self.width), MATRIX)
+            req["dkv_weight"] = WeightRequest((self.rank + self.rot_dim, self.width), MATRIX)
             req["dkv_norm"] = WeightRequest((self.rank,), VECTOR)
         return req
+
+    def token_matrix_elements(self) -> int:
+        if self.in_weight is None:
+            return 0
+        return self.in_weight.numel() + self.uk_folded.numel() + self.uv_heads.numel() + self.out_weight.numel()
 
     def bind(self, tensors):
         super().bind(tensors)
         # the products that read h as one: queries, gate and (where this layer makes it) the latent
         names = ["q_weight", "gate_weight"] + (["dkv_weight"] if self.makes_latent else [])
-        self.in_weight = torch.cat([tensors[n] for n in names], dim=0).contiguous()
+        stacked = [tensors[n] for n in names]
+        rows = sum(t.shape[0] for t in stacked)
+        if self.rot_dim and rows % 16:      # rows of the products' output start 16 bytes apart
+            stacked.append(torch.zeros((16 - rows % 16, self.width), dtype=stacked[0].dtype, device=stacked[0].device))
+        self.in_weight = torch.cat(stacked, dim=0).contiguous()
         views, at = {}, 0
         for n in names:
             rows = tensors[n].shape[0]
             views[n] = self.in_weight[at:at + rows]
             setattr(self, n, views[n])
             at += rows
-        # per head: Wuk_a^T as [rank, D] (so that folding a query is a product with a matrix stored
-        # [out, in]) and Wuv_a as [E, rank]
-        self.uk_folded = self.uk_weight.view(self.n_head, self.head_dim, self.rank).transpose(1, 2).contiguous()
-        self.uv_heads = self.uv_weight.view(self.n_head, self.value_dim, self.rank)
-        self.uk_weight = self.uk_folded.transpose(1, 2)
+        # per head: Wuk_a^T as [row, D (+ P)] (so that folding a query is a product with a matrix stored
+        # [out, in]; the rotated part of a query passes through an identity block) and Wuv_a as [E, row]
+        H, D, P, R = self.n_head, self.head_dim, self.rot_dim, self.rank
+        uk_t = self.uk_weight.view(H, D, R).transpose(1, 2)
+        if P:
+            folded = torch.zeros((H, self.row, D + P), dtype=uk_t.dtype, device=uk_t.device)
+            folded[:, :R, :D] = uk_t
+            folded[:, R:R + P, D:] = torch.eye(P, dtype=uk_t.dtype, device=uk_t.device)
+            self.uk_folded = folded
+            uv = torch.zeros((H, self.value_dim, self.row), dtype=uk_t.dtype, device=uk_t.device)
+            uv[:, :, :R] = self.uv_weight.view(H, self.value_dim, R)
+            self.uv_heads = uv
+            self.uk_weight = folded[:, :R, :D].transpose(1, 2)
+            views["uv_weight"] = uv[:, :, :R]
+            self.uv_weight = views["uv_weight"]
+        else:
+            self.uk_folded = uk_t.contiguous()
+            self.uv_heads = self.uv_weight.view(H, self.value_dim, R)
+            self.uk_weight = self.uk_folded.transpose(1, 2)
         views["uk_weight"] = self.uk_weight
         return views
 
     def cache_need(self) -> KVNeed:
-        return KVNeed(1, self.rank, self.window, joint=True)
+        return KVNeed(1, self.row, self.window, joint=True)
 
     def forward_add(self, ctx: StepContext, h, x: torch.Tensor, binding: CacheBinding,
                     position: PositionEncoding) -> None:
@@ -216,7 +260,8 @@ class LatentAttention(Mixer):
         fast = not ctx.exact
         z = ws.get("latent_in", n, self.in_weight.shape[0], ctx.dtype)
         split = self.q_width + self.g_width
-        if self.makes_latent and n > self.JOINT_PRODUCT_MAX_ROWS and n * split > self.JOINT_PRODUCT_MAX_WORK:
+        if (self.makes_latent and not self.rot_dim and n > self.JOINT_PRODUCT_MAX_ROWS
+                and n * split > self.JOINT_PRODUCT_MAX_WORK):
             # many rows: the few latent columns on top of queries and gate would start another
             # round of the tiled kernel's tiles (17 x 16 tiles of 128 x 256 on 256 compute units
             # where 16 x 16 fit), so the latent gets a small product of its own
@@ -227,16 +272,23 @@ class LatentAttention(Mixer):
             linear(ctx, h, self.in_weight, None, z, n)
         group = ctx.groups[binding.group]
         pool = group.k_pools[binding.index]
-        if self.makes_latent:
-            kernels.rms_norm_store(z[:, self.q_width + self.g_width:], self.dkv_norm, self.eps, pool,
-                                   group.slot_mapping, n)
-        q_lat = ws.get("latent_q", n, self.n_head * self.rank, ctx.dtype)
+        if self.rot_dim:
+            # the queries' rotated parts in place; the normed latent and the rotated key part into the pages
+            kernels.latent_prepare(z, 0, self.n_head, self.head_dim, self.rot_dim, ctx.positions,
+                                   self.rotation.frequencies(z.device), n, getattr(self.rotation, "magnitude", 1.0),
+                                   c_off=split, rank=self.rank, gain=self.dkv_norm if self.makes_latent else None,
+                                   eps=self.eps, pool=pool if self.makes_latent else None,
+                                   slot_mapping=group.slot_mapping if self.makes_latent else None)
+        elif self.makes_latent:
+            kernels.rms_norm_store(z[:, split:], self.dkv_norm, self.eps, pool, group.slot_mapping, n)
+        q_lat = ws.get("latent_q", n, self.n_head * self.row, ctx.dtype)
         kernels.heads_linear(z, self.uk_folded, q_lat, n, fast=fast)
-        o_lat = ws.get("latent_o", n, self.n_head * self.rank, ctx.dtype)
+        o_lat = ws.get("latent_o", n, self.n_head * self.row, ctx.dtype)
+        gate = z[:, self.q_width:split]
         attention_ops.paged_attention(ctx, q_lat, o_lat, pool, pool, group, self.n_head, self.scale, self.window,
-                                      sinks=self.sink)
-        y = ws.get("attn_out", n, self.g_width, ctx.dtype)
-        kernels.heads_linear(o_lat, self.uv_heads, y, n, gate=z[:, self.q_width:self.q_width + self.g_width], fast=fast)
+                                      sinks=self.sink, gate=gate if self.head_gate else None)
+        y = ws.get("attn_out", n, self.y_width, ctx.dtype)
+        kernels.heads_linear(o_lat, self.uv_heads, y, n, gate=None if self.head_gate else gate, fast=fast)
         linear_add(ctx, y, self.out_weight, None, x, n)
 
 
@@ -267,7 +319,15 @@ class GatedAttention(Mixer):
     into the residual.  With `conv_taps` = J > 1 the projected q, k and v pass a causal convolution over
     time first, channel by channel (weights [channels, J], the last tap on the current token, zeros
     before the sequence's start), whose last J - 1 inputs are kept per request beside the pages.  With
-    `window` = w > 0 a query sees only the keys at the last w positions, its own included.
+    `window` = w > 0 a query sees only the keys at the last w positions, its own included, and with
+    `keep_first` = f also those at positions below f (which keep their true positions).  Further options:
+    `qk_norm_weights` "head" or "whole": instead of the unit norm behind the rotation, an RMS norm with weights
+    (eps `qk_norm_eps`) *before* the rotation, head by head with one weight vector [D] that the query heads share
+    and one for the key heads, or over all of a token's query channels at once (and all of its key channels) with
+    weights as long as the projection; `values_from_keys`: there is no Wv, a key head's values are its keys as
+    projected (before norm and rotation), so E = D; `score_bias`: no softmax, a visible key's weight is
+    sigmoid(score + b_a) with a number per head (the tensor `score_bias`), not normalised over the keys;
+    `out_bias`: the output projection has a bias.
 
     The cache keeps keys and values in pages of one head size, so both are laid out with
     max(D, E) channels a head (rounded up to what the bfloat16 attention kernels take), the
@@ -279,7 +339,9 @@ class GatedAttention(Mixer):
     def __init__(self, width: int, n_head: int, n_kv_head: int, head_dim: int, value_dim: int, scale: float,
                  bias: bool = False, rotary: Optional[dict] = None, qk_norm_eps: Optional[float] = None,
                  softcap: float = 0.0, head_gate: bool = False, value_mix: Optional[str] = None,
-                 share: str = "values", conv_taps: int = 0, window: int = 0) -> None:
+                 share: str = "values", conv_taps: int = 0, window: int = 0, keep_first: int = 0,
+                 qk_norm_weights: Optional[str] = None, values_from_keys: bool = False, score_bias: bool = False,
+                 out_bias: bool = False) -> None:
         self.width, self.n_head, self.n_kv_head = int(width), int(n_head), int(n_kv_head)
         self.head_dim, self.value_dim, self.scale = int(head_dim), int(value_dim), float(scale)
         self.has_bias, self.has_gate = bool(bias), bool(head_gate)
@@ -296,6 +358,17 @@ class GatedAttention(Mixer):
             raise ValueError("n_head must be a multiple of n_kv_head")
         if self.rotation is not None and self.rotation.dims > self.head_dim:
             raise ValueError(f"rotation over {self.rotation.dims} channels of heads of {self.head_dim}")
+        self.keep_first = int(keep_first or 0) if self.window else 0
+        if int(keep_first or 0) < 0:
+            raise ValueError("keep_first must not be negative")
+        if qk_norm_weights not in (None, "head", "whole") or (qk_norm_weights and self.qk_norm_eps is None):
+            raise ValueError("qk_norm_weights is None, 'head' or 'whole', and needs qk_norm_eps")
+        self.qk_norm_weights = qk_norm_weights
+        self.values_from_keys, self.has_score_bias, self.has_out_bias = bool(values_from_keys), bool(score_bias), bool(out_bias)
+        if self.values_from_keys and (self.value_dim != self.head_dim or self.value_mix is not None or self.conv_taps > 1):
+            raise ValueError("values that are the keys have the keys' size, and are neither mixed nor convolved")
+        if self.has_score_bias and self.softcap > 0.0:
+            raise ValueError("sigmoid weights take no score cap")
         size = max(self.head_dim, self.value_dim)
         self.head_stride = -(-size // 32) * 32 if size <= 128 else -(-size // 8) * 8
         if self.head_stride > 512:
@@ -303,21 +376,31 @@ class GatedAttention(Mixer):
         s = self.head_stride
         self.q_off, self.k_off = 0, self.n_head * s
         self.v_off = self.k_off + self.n_kv_head * s
-        self.g_off = self.v_off + self.n_kv_head * s
+        self.g_off = self.v_off + (0 if self.values_from_keys else self.n_kv_head * s)
         self.in_rows = -(-(self.g_off + (self.n_head if self.has_gate else 0)) // 16) * 16
         self.in_weight = self.in_bias = self.out_padded = self.conv_weight = None
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
         H, G, D, E, W = self.n_head, self.n_kv_head, self.head_dim, self.value_dim, self.width
         req = {"q_weight": WeightRequest((H * D, W), MATRIX), "k_weight": WeightRequest((G * D, W), MATRIX),
-               "v_weight": WeightRequest((G * E, W), MATRIX), "out_weight": WeightRequest((W, H * E), MATRIX)}
+               "out_weight": WeightRequest((W, H * E), MATRIX)}
+        if not self.values_from_keys:
+            req["v_weight"] = WeightRequest((G * E, W), MATRIX)
+        if self.qk_norm_weights is not None:
+            whole = self.qk_norm_weights == "whole"
+            req.update(q_norm=WeightRequest((H * D if whole else D,), VECTOR), k_norm=WeightRequest((G * D if whole else D,), VECTOR))
+        if self.has_score_bias:
+            req["score_bias"] = WeightRequest((H,), VECTOR)
+        if self.has_out_bias:
+            req["out_bias"] = WeightRequest((W,), VECTOR)
         if self.conv_taps > 1:
             J = self.conv_taps
             req.update(q_conv=WeightRequest((H * D, J), VECTOR), k_conv=WeightRequest((G * D, J), VECTOR),
                        v_conv=WeightRequest((G * E, J), VECTOR))
         if self.has_bias:
-            req.update(q_bias=WeightRequest((H * D,), VECTOR), k_bias=WeightRequest((G * D,), VECTOR),
-                       v_bias=WeightRequest((G * E,), VECTOR))
+            req.update(q_bias=WeightRequest((H * D,), VECTOR), k_bias=WeightRequest((G * D,), VECTOR))
+            if not self.values_from_keys:
+                req["v_bias"] = WeightRequest((G * E,), VECTOR)
         if self.has_gate:
             req["gate_weight"] = WeightRequest((H, W), MATRIX)
         if self.value_mix is not None:
@@ -338,7 +421,8 @@ class GatedAttention(Mixer):
 
         place("q_weight", self.q_off, H, D)
         place("k_weight", self.k_off, G, D)
-        place("v_weight", self.v_off, G, E)
+        if not self.values_from_keys:
+            place("v_weight", self.v_off, G, E)
         if self.has_gate:
             joint[self.g_off:self.g_off + H].copy_(tensors["gate_weight"])
             views["gate_weight"] = joint[self.g_off:self.g_off + H]
@@ -347,6 +431,8 @@ class GatedAttention(Mixer):
             bias = torch.zeros(self.in_rows, dtype=torch.float32, device=q.device)
             for name, at, heads, size in (("q_bias", self.q_off, H, D), ("k_bias", self.k_off, G, D),
                                           ("v_bias", self.v_off, G, E)):
+                if name not in tensors:
+                    continue
                 bias[at:at + heads * s].view(heads, s)[:, :size].copy_(tensors[name].view(heads, size))
             self.in_bias = bias
         if self.conv_taps > 1:
@@ -366,7 +452,7 @@ class GatedAttention(Mixer):
         return views
 
     def cache_need(self) -> KVNeed:
-        return KVNeed(self.n_kv_head, self.head_stride, self.window,
+        return KVNeed(self.n_kv_head, self.head_stride, self.window, keep_first=self.keep_first,
                       state_numel=(self.conv_taps - 1) * self.g_off if self.conv_taps > 1 else 0)
 
     def token_matrix_elements(self) -> int:
@@ -399,12 +485,17 @@ class GatedAttention(Mixer):
                            positions=ctx.positions,
                            freq=self.rotation.frequencies(z.device) if self.rotation is not None else None,
                            norm_eps=self.qk_norm_eps, mix_lambda=self.mix if mode == 2 else None, v_other=other,
-                           mix_mode=mode, k_pool=k_pool, v_pool=v_pool, slot_mapping=group.slot_mapping)
+                           mix_mode=mode, k_pool=k_pool, v_pool=v_pool, slot_mapping=group.slot_mapping,
+                           norm=self.qk_norm_weights, q_norm_weight=self.q_norm if self.qk_norm_weights else None,
+                           k_norm_weight=self.k_norm if self.qk_norm_weights else None,
+                           values_from_keys=self.values_from_keys,
+                           rot_magnitude=getattr(self.rotation, "magnitude", 1.0))
         y = ws.get("attn_out", n, self.n_head * s, ctx.dtype)
         # (the gate per head is applied by the attention kernel as it stores a head's output)
         attention_ops.paged_attention(ctx, z, y, k_pool, v_pool, group, self.n_head, self.scale, self.window,
-                                      softcap=self.softcap, gate=gate_rows[:, self.g_off:] if self.has_gate else None)
-        linear_add(ctx, y, self.out_padded, None, x, n)
+                                      softcap=self.softcap, gate=gate_rows[:, self.g_off:] if self.has_gate else None,
+                                      keep_first=self.keep_first, score_bias=self.score_bias if self.has_score_bias else None)
+        linear_add(ctx, y, self.out_padded, self.out_bias if self.has_out_bias else None, x, n)
 
 
 @register_mixer("decay_state")

@@ -25,6 +25,9 @@ from .base import (ARRANGEMENTS, CacheBinding, EMBEDDINGS, FEED_FORWARDS, HEADS,
                    POSITIONS, Part, PartSpec, StateNeed, StepContext, WeightRequest)
 
 
+# the name under which a run's bindings hold the state pool of the layer's arrangement, if it keeps any
+ARRANGEMENT_ROLE = _block.STATE_ROLE
+
 # categories of a layer's parts, and the registry of each
 _LAYER_REGISTRIES = {"norm": NORMS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS}
 
@@ -96,6 +99,7 @@ class CacheGroupSpec:
     window: int        # what the pages must keep: the widest window among the runs that write or read them
     n_pools: int       # caches (one per writing run) in the group
     joint: bool = False   # keys and values are one tensor
+    keep_first: int = 0   # with a window: the first positions whose pages stay (the most any run of the group keeps)
 
 
 @dataclass
@@ -107,7 +111,8 @@ class CacheLayout:
     @property
     def bindings(self) -> List[CacheBinding]:
         """One binding per run, for models whose layers have exactly one mixer each."""
-        return [next(iter(b.values())) if len(b) == 1 else None for b in self.run_bindings]
+        mixers = [[v for role, v in b.items() if role != ARRANGEMENT_ROLE] for b in self.run_bindings]
+        return [m[0] if len(m) == 1 else None for m in mixers]
 
 
 @dataclass(frozen=True)
@@ -118,6 +123,7 @@ class KVRun:
     head_dim: int
     window: int
     tensors: int = 2      # cached tensors a key position costs: keys and values, or one joint latent
+    keep_first: int = 0   # first positions seen beside the window
 
 
 @dataclass(frozen=True)
@@ -139,7 +145,7 @@ class ModelCost:
         kv = 0.0
         for run in self.kv_runs:
             for c in context_lens:
-                reach = min(c, run.window) if run.window else c
+                reach = min(c, run.window + run.keep_first) if run.window else c
                 kv += reach * run.tensors * run.n_kv_head * run.head_dim * cache_itemsize
         return self.whole_tensor_bytes + n_tokens * self.table_row_bytes + kv + 4.0 * self.state_floats * len(context_lens)
 
@@ -150,7 +156,7 @@ class ModelCost:
         flops = 2.0 * n * self.run_matrix_elements + 2.0 * n_logit_rows * self.head_matrix_elements
         for run in self.kv_runs:
             for t in prompt_lens:
-                seen = sum(min(i + 1, run.window) if run.window else i + 1 for i in range(t))
+                seen = sum(min(i + 1, run.window + run.keep_first) if run.window else i + 1 for i in range(t))
                 flops += 4.0 * seen * run.n_head * run.head_dim
         return flops
 
@@ -282,17 +288,18 @@ class DecoderModel:
                 need = part.cache_need() if hasattr(part, "cache_need") else None
                 if isinstance(need, KVNeed):
                     kv_runs.append(KVRun(int(getattr(part, "n_head", need.n_kv_head)), need.n_kv_head,
-                                         need.head_dim, need.window, 1 if need.joint else 2))
+                                         need.head_dim, need.window, 1 if need.joint else 2, need.keep_first))
                     state_floats += int(need.state_numel)
                 elif isinstance(need, StateNeed):
                     state_floats += int(need.numel)
+            state_floats += int(getattr(layer.arrangement, "state_numel", lambda: 0)())
         return ModelCost(sum(size(name) for name in whole), row_bytes, run_elements, matrices(self.head),
                          tuple(kv_runs), state_floats)
 
     # ------------------------------------------------------------------ cache
     def _plan_cache(self) -> CacheLayout:
         groups: List[CacheGroupSpec] = []
-        keys: List[Tuple[int, int, int, bool]] = []
+        keys: List[Tuple[int, int, int, bool, int]] = []
         state_numels: List[int] = []
         run_bindings: List[Dict[str, CacheBinding]] = []
 
@@ -306,7 +313,7 @@ class DecoderModel:
 
         # What a writing run's pages must keep: the widest window among itself and the runs that read
         # its cache (each masks with its own window; 0, all keys, is the widest).
-        reach: Dict[Tuple[int, str], int] = {}
+        reach: Dict[Tuple[int, str], Tuple[int, int]] = {}      # (window, first positions kept beside it)
         for i, run in enumerate(self.spec.order):
             for role in self.spec.layers[run.layer].roles("mixer"):
                 need = need_of(i, role)
@@ -314,7 +321,12 @@ class DecoderModel:
                     continue
                 key = (i if run.reads_cache_of is None else run.reads_cache_of, role)
                 seen = reach.get(key)
-                reach[key] = need.window if seen is None else (0 if 0 in (seen, need.window) else max(seen, need.window))
+                if seen is None:
+                    reach[key] = (need.window, need.keep_first if need.window else 0)
+                elif 0 in (seen[0], need.window):
+                    reach[key] = (0, 0)
+                else:
+                    reach[key] = (max(seen[0], need.window), max(seen[1], need.keep_first))
 
         for i, run in enumerate(self.spec.order):
             layer_spec = self.spec.layers[run.layer]
@@ -328,22 +340,28 @@ class DecoderModel:
                         raise ValueError(f"run {i} cannot read the cache of run {run.reads_cache_of}: different needs")
                     bindings[role] = CacheBinding("kv", src.group, src.index, writes=False)
                 elif isinstance(need, KVNeed):
-                    key = (need.n_kv_head, need.head_dim, reach[(i, role)], need.joint)
+                    key = (need.n_kv_head, need.head_dim, reach[(i, role)][0], need.joint, reach[(i, role)][1])
                     if key not in keys:
                         keys.append(key)
-                        groups.append(CacheGroupSpec(key[0], key[1], key[2], 0, key[3]))
+                        groups.append(CacheGroupSpec(key[0], key[1], key[2], 0, key[3], key[4]))
                     g = keys.index(key)
                     state = -1
                     if need.state_numel:
                         state = len(state_numels)
                         state_numels.append(int(need.state_numel))
                     bindings[role] = CacheBinding("kv", g, groups[g].n_pools, writes=True, state=state)
-                    groups[g] = CacheGroupSpec(key[0], key[1], key[2], groups[g].n_pools + 1, key[3])
+                    groups[g] = CacheGroupSpec(key[0], key[1], key[2], groups[g].n_pools + 1, key[3], key[4])
                 elif isinstance(need, StateNeed):
                     bindings[role] = CacheBinding("state", -1, len(state_numels), writes=True)
                     state_numels.append(int(need.numel))
                 else:
                     bindings[role] = CacheBinding("none")
+            # an arrangement may keep float32 values per request of its own (what it carries from a token to the
+            # next): a state pool like a mixer's, under the role name "arrangement"
+            kept = int(getattr(self.layers[run.layer].arrangement, "state_numel", lambda: 0)())
+            if kept:
+                bindings[ARRANGEMENT_ROLE] = CacheBinding("state", -1, len(state_numels), writes=True)
+                state_numels.append(kept)
             run_bindings.append(bindings)
         if not groups:
             # a model that keeps no keys and values (state mixers only): one group without pools, so that the
