@@ -147,6 +147,19 @@ def window_with_first(T: int, size: int, keep_first: int) -> torch.Tensor:
     return (j <= i) & ((i - j < size) | (j < keep_first))
 
 
+def attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, seen: torch.Tensor,
+           score_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q, k [T, H, D], v [T, H, E], seen [T, T] (query i sees key j).  Weights: a softmax of the scaled scores over
+    the keys seen, or with score_bias [H] sigmoid(score + score_bias[h]) for every key seen, not normalised.
+    Returns [T, H, E]."""
+    s = torch.einsum("ihd,jhd->hij", q, k) * scale
+    if score_bias is None:
+        w = torch.softmax(s.masked_fill(~seen[None], -math.inf), dim=-1)
+    else:
+        w = sigmoid(s + score_bias[:, None, None]) * seen[None]
+    return torch.einsum("hij,jhe->ihe", w, v)
+
+
 def latent_attention(h: torch.Tensor, t: Dict[str, torch.Tensor], p: str, m: dict, eps: float,
                      shared: Optional[Tuple[torch.Tensor, torch.Tensor]]) -> Tuple[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
     """Returns the mixer's output and (latents [T, R], rotated shared key part [T, P]), which a later layer may use."""
@@ -182,10 +195,9 @@ def sigmoid_attention(h: torch.Tensor, t: Dict[str, torch.Tensor], p: str, m: di
     q = _r(rotate_half(q.view(T, H, D), dims, freq, mag))
     k = _r(rotate_half(k.view(T, G, D), dims, freq, mag)).repeat_interleave(H // G, dim=1)
     v = v.repeat_interleave(H // G, dim=1)
-    s = torch.einsum("ihd,jhd->hij", q, k) * m["scale"]
-    w = sigmoid(s + t[p + "pb"][:, None, None])
-    w = w * window_with_first(T, m["mask"]["size"], m["mask"]["keep_first"])[None]
-    y = torch.einsum("hij,jhe->ihe", w, v)
+    mask = m.get("mask")
+    seen = window_with_first(T, mask["size"], mask.get("keep_first", 0)) if mask else causal(T)
+    y = attend(q, k, v, m["scale"], seen, t[p + "pb"])
     return lin(_r(y.reshape(T, H * E)), t[p + "o"], t[p + "o.b"])
 
 
@@ -199,10 +211,7 @@ def keyed_value_attention(h: torch.Tensor, t: Dict[str, torch.Tensor], p: str, m
     dims, freq, mag = rotation_of(m["rot"])
     q = _r(rotate_half(unit_rms(q, eps) * t[p + "q.norm"], dims, freq, mag))
     k = _r(rotate_half(unit_rms(k, eps) * t[p + "k.norm"], dims, freq, mag)).repeat_interleave(H // G, dim=1)
-    s = torch.einsum("ihd,jhd->hij", q, k) * m["scale"]
-    s = s.masked_fill(~causal(T)[None], -math.inf)
-    w = torch.softmax(s, dim=-1)
-    y = torch.einsum("hij,jhe->ihe", w, v)
+    y = attend(q, k, v, m["scale"], causal(T))
     return lin(_r(y.reshape(T, H * m["vdim"])), t[p + "o"])
 
 
@@ -234,3 +243,13 @@ def forward(cfg: dict, t: Dict[str, torch.Tensor], ids: List[int], layers_out: O
             layers_out.append(x.clone())
     h = unit_rms(x, eps) * (1.0 + t["final.norm"])
     return lin(h, t["head"])
+
+
+def greedy(cfg: dict, t: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:
+    """n_new tokens chosen greedily (the lowest index among equals), the whole sequence computed anew each time."""
+    seq, out = list(prompt), []
+    for _ in range(n_new):
+        tok = int(torch.argmax(forward(cfg, t, seq)[-1]))
+        out.append(tok)
+        seq.append(tok)
+    return out
