@@ -343,13 +343,38 @@ def rilavik_like(layers, width, heads, vocab):
     return {"architecture": "Rilavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": out}
 
 
-COMPARED = {"viperax": viperax_like, "bobevik": bobevik_like, "rilavik": rilavik_like}
+def nutitar_like(layers, width, heads, vocab):
+    """A Nutitar config.json of a GPT-2-style model's size: the same layers, width, heads and vocabulary, heads
+    of 128 channels; the layer types in turn (attention_2, latent_attention, attention, attention; two layers:
+    latent_attention, attention); a dense feed-forward with a hidden size of 4 width in every layer, as the
+    GPT-2 MLP.  Grouped layers have a quarter as many key/value heads as heads; the windowed ones see 512
+    positions beside the first 64; a latent is 96 values beside a rotated key part of 32 (a cached row of 128)."""
+    kinds = ["latent_attention", "attention"] if layers <= 2 else ["attention_2", "latent_attention", "attention", "attention"]
+    kv = max(heads // 4, 1)
+    out = []
+    for i in range(layers):
+        kind = kinds[i % len(kinds)]
+        if kind == "latent_attention":
+            mixer = {"heads": heads, "dim": 96, "rot_dim": 32, "vdim": 128, "kv_rank": 96, "scale": 128 ** -0.5,
+                     "rot": {"dims": 32, "base": 1e6, "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+        elif kind == "attention":
+            mixer = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "mask": {"size": 512, "keep_first": 64}, "rot": {"dims": 64, "base": 5e5}}
+        else:
+            mixer = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "rot": {"dims": 128, "base": 1e4, "scaling": {"factor": 8.0, "original": 8192, "low": 1.0, "high": 4.0}}}
+        out.append({"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": 4 * width}})
+    return {"architecture": "Nutitar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+            "embedding": {"scale": 1.0}, "layers": out}
+
+
+COMPARED = {"viperax": viperax_like, "bobevik": bobevik_like, "rilavik": rilavik_like, "nutitar": nutitar_like}
 # the model a design is measured beside: the GPT-2-style model, or the design nearest to it
 BESIDE = {"rilavik": "bobevik"}
 
 
 def compare_run(args, name):
-    """--compare viperax | bobevik | rilavik: prefill (2 prompts of 1,024 tokens as one step) and decode
+    """--compare viperax | bobevik | rilavik | nutitar: prefill (2 prompts of 1,024 tokens as one step) and decode
     (batch 8, by the default run's timing rule, fewer blocks) of that design beside the GPT-2-style model
     (Rilavik: beside Bobevik, the nearest design) at equal layers, width, heads and vocabulary, random
     weights, at COMPARE_SIZES.  One JSON line."""

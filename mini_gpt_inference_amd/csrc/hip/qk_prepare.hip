@@ -24,8 +24,9 @@
 #include "launchers.h"
 
 #define QKP_MAX_DIM 512
+#define QKP_MAX_WAVES 16   // a wave a head at a time: as many waves as the token has query and key heads, up to these
 
-__global__ __launch_bounds__(256) void qk_prepare_kernel(
+__global__ __launch_bounds__(1024) void qk_prepare_kernel(
     void* __restrict__ z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head, int n_kv_head,
     int head_dim, int value_dim, int head_stride, const int* __restrict__ positions, const float* __restrict__ freq, int rot_dims,
     float norm_eps, const float* __restrict__ mix_lambda, void* __restrict__ v_other, long ld_other, int mix_mode,
@@ -33,14 +34,14 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     int n_tokens, int norm_mode, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, int v_from_k,
     float rot_mag) {
   __shared__ float cos_s[QKP_MAX_DIM / 2], sin_s[QKP_MAX_DIM / 2];
-  __shared__ float head_s[4][QKP_MAX_DIM];
-  __shared__ float red_s[8];
+  __shared__ float head_s[QKP_MAX_WAVES][QKP_MAX_DIM];
+  __shared__ float red_s[2 * QKP_MAX_WAVES];
   const int n = blockIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n_waves = blockDim.x >> 6;
   const int half = rot_dims / 2;
   if (freq) {
     const float p = (float)positions[n];
-    for (int i = threadIdx.x; i < half; i += 256) {
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
       const float a = p * freq[i];
       cos_s[i] = cosf(a) * rot_mag;
       sin_s[i] = sinf(a) * rot_mag;
@@ -50,12 +51,12 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   float whole_q = 1.0f, whole_k = 1.0f;   // norm_mode 2: what all query (key) channels of the token are multiplied by
   if (norm_mode == 2) {
     float sq = 0.f, sk = 0.f;
-    for (int i = threadIdx.x; i < n_head * head_dim; i += 256) {
+    for (int i = threadIdx.x; i < n_head * head_dim; i += blockDim.x) {
       const int hh = i / head_dim;
       const float v = load_f(z, dtype, row + q_off + (long)hh * head_stride + (i - hh * head_dim));
       sq = fmaf(v, v, sq);
     }
-    for (int i = threadIdx.x; i < n_kv_head * head_dim; i += 256) {
+    for (int i = threadIdx.x; i < n_kv_head * head_dim; i += blockDim.x) {
       const int hh = i / head_dim;
       const float v = load_f(z, dtype, row + k_off + (long)hh * head_stride + (i - hh * head_dim));
       sk = fmaf(v, v, sk);
@@ -64,18 +65,23 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     sk = wave_sum(sk);
     if (lane == 0) {
       red_s[wave] = sq;
-      red_s[4 + wave] = sk;
+      red_s[QKP_MAX_WAVES + wave] = sk;
     }
     __syncthreads();
-    whole_q = 1.0f / sqrtf(((red_s[0] + red_s[1]) + (red_s[2] + red_s[3])) / (float)(n_head * head_dim) + norm_eps);
-    whole_k = 1.0f / sqrtf(((red_s[4] + red_s[5]) + (red_s[6] + red_s[7])) / (float)(n_kv_head * head_dim) + norm_eps);
+    sq = sk = 0.f;
+    for (int w = 0; w < n_waves; ++w) {      // in wave order, the same sum in every thread
+      sq += red_s[w];
+      sk += red_s[QKP_MAX_WAVES + w];
+    }
+    whole_q = 1.0f / sqrtf(sq / (float)(n_head * head_dim) + norm_eps);
+    whole_k = 1.0f / sqrtf(sk / (float)(n_kv_head * head_dim) + norm_eps);
   }
   __syncthreads();
   const int slot = slot_mapping ? slot_mapping[n] : -1;
   const long page = slot >= 0 ? slot / page_size : 0;
   const int off = slot >= 0 ? slot - (int)page * page_size : 0;
   float* s = head_s[wave];
-  for (int hh = wave; hh < n_head + n_kv_head; hh += 4) {
+  for (int hh = wave; hh < n_head + n_kv_head; hh += n_waves) {
     const bool is_q = hh < n_head;
     const int g = is_q ? hh : hh - n_head;
     if (!is_q && !kpool) continue;
@@ -155,7 +161,8 @@ extern "C" int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_of
   if (norm_mode < 0 || norm_mode > 2 || (norm_mode && !(norm_eps >= 0.f)) || (v_from_k && (mix_mode || value_dim != head_dim)))
     return MGPT_ERR_BAD_SHAPE;
   if (norm_mode && (!q_norm_w || !k_norm_w)) return MGPT_ERR_NULL;
-  hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(256), 0, stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
+  const int waves = n_head + n_kv_head < QKP_MAX_WAVES ? (n_head + n_kv_head < 4 ? 4 : n_head + n_kv_head) : QKP_MAX_WAVES;
+  hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(64 * waves), 0, stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
                      n_kv_head, head_dim, value_dim, head_stride, positions, rot_dims ? freq : nullptr, rot_dims, norm_eps, mix_lambda,
                      v_other, ld_other, mix_mode, kpool, vpool, slot_mapping, page_size, n_tokens, norm_mode, q_norm_w, k_norm_w,
                      v_from_k, rot_mag);

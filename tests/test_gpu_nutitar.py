@@ -79,14 +79,14 @@ def test_xielu(dtype, n, hidden):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("width", [40, 256, 1030])
-def test_norm_and_token_shift_keep_a_row_per_request(dtype, width):
+@pytest.mark.parametrize("width,pad", [(40, 3), (40, 0), (256, 4), (1030, 2), (2048, 0), (3076, 8)])
+def test_norm_and_token_shift_keep_a_row_per_request(dtype, width, pad):
     """Four requests of 70, 1, 32 and 33 tokens: whole, in portions cut anywhere, and one token a step (where one
     kernel norms, shifts and keeps); the kept rows start as NaN, and the slots are used a second time by other
     sequences.  Beside the shift: the pending addition is made, the sums are cleared, h is the norm."""
     g = torch.Generator().manual_seed(width)
     gain, shift = _rnd(g, width, scale=0.2), torch.rand(width, generator=g)
-    state = torch.full((6, width + 3), float("nan"), device=DEV)
+    state = torch.full((6, width + pad), float("nan"), device=DEV)
     for trial in range(2):
         x0, y0 = _rnd(g, N_ROWS, width, scale=3.0), _rnd(g, N_ROWS, width)
         xs = _d(x0) + 0.3 * _d(y0)
