@@ -34,8 +34,8 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
     int n_tokens, int norm_mode, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, int v_from_k,
     float rot_mag) {
   __shared__ float cos_s[QKP_MAX_DIM / 2], sin_s[QKP_MAX_DIM / 2];
-  __shared__ float head_s[QKP_MAX_WAVES][QKP_MAX_DIM];
   __shared__ float red_s[2 * QKP_MAX_WAVES];
+  extern __shared__ float head_s[];    // [waves][head_dim]: the head a wave is working on
   const int n = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n_waves = blockDim.x >> 6;
   const int half = rot_dims / 2;
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
   const int slot = slot_mapping ? slot_mapping[n] : -1;
   const long page = slot >= 0 ? slot / page_size : 0;
   const int off = slot >= 0 ? slot - (int)page * page_size : 0;
-  float* s = head_s[wave];
+  float* s = head_s + wave * head_dim;
   for (int hh = wave; hh < n_head + n_kv_head; hh += n_waves) {
     const bool is_q = hh < n_head;
     const int g = is_q ? hh : hh - n_head;
@@ -161,8 +161,11 @@ extern "C" int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_of
   if (norm_mode < 0 || norm_mode > 2 || (norm_mode && !(norm_eps >= 0.f)) || (v_from_k && (mix_mode || value_dim != head_dim)))
     return MGPT_ERR_BAD_SHAPE;
   if (norm_mode && (!q_norm_w || !k_norm_w)) return MGPT_ERR_NULL;
-  const int waves = n_head + n_kv_head < QKP_MAX_WAVES ? (n_head + n_kv_head < 4 ? 4 : n_head + n_kv_head) : QKP_MAX_WAVES;
-  hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(64 * waves), 0, stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
+  // few tokens (a decode step): a wave per head, so that a token's heads are done side by side; many tokens: four
+  // waves a token, and more tokens at a time on a compute unit
+  int waves = 4;
+  if (n_tokens < 64 && n_head + n_kv_head > 4) waves = n_head + n_kv_head < QKP_MAX_WAVES ? n_head + n_kv_head : QKP_MAX_WAVES;
+  hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(64 * waves), waves * head_dim * sizeof(float), stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
                      n_kv_head, head_dim, value_dim, head_stride, positions, rot_dims ? freq : nullptr, rot_dims, norm_eps, mix_lambda,
                      v_other, ld_other, mix_mode, kpool, vpool, slot_mapping, page_size, n_tokens, norm_mode, q_norm_w, k_norm_w,
                      v_from_k, rot_mag);

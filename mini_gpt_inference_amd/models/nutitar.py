@@ -63,7 +63,7 @@ class MixerConfig:
     dim: int
     vdim: int
     scale: float
-    rot: Rotation
+    rot: Optional[Rotation]            # None (a grouped layer without a rot entry): queries and keys are not rotated
     kv_heads: int = 0                   # attention, attention_2
     window: int = 0                     # attention: mask.size; 0: every earlier key
     keep_first: int = 0                 # attention: mask.keep_first
@@ -135,7 +135,7 @@ def _mixer(where: str, kind: str, m: Mapping[str, Any]) -> MixerConfig:
     kv_heads = _positive(f"{where} kv_heads", m.get("kv_heads"))
     if heads % kv_heads:
         raise ConfigError(f"{where}: heads must be a multiple of kv_heads")
-    rot = _rotation(where, m.get("rot"), dim)
+    rot = _rotation(where, m["rot"], dim) if m.get("rot") is not None else None
     window = keep_first = 0
     mask = m.get("mask")
     if mask is not None:
@@ -188,7 +188,9 @@ def config_to_json(cfg: NutitarConfig) -> Dict[str, Any]:
     layers = []
     for layer in cfg.layers:
         m = layer.mixer
-        mixer: Dict[str, Any] = {"dim": m.dim, "heads": m.heads, "rot": _rotation_json(m.rot), "scale": m.scale, "vdim": m.vdim}
+        mixer: Dict[str, Any] = {"dim": m.dim, "heads": m.heads, "scale": m.scale, "vdim": m.vdim}
+        if m.rot is not None:
+            mixer["rot"] = _rotation_json(m.rot)
         if layer.type == "latent_attention":
             mixer.update(kv_rank=m.kv_rank, rot_dim=m.rot_dim)
             if m.kv_from is not None:
@@ -223,7 +225,7 @@ def model_spec(cfg: NutitarConfig) -> ModelSpec:
         names = {"q_weight": p + "q", "k_weight": p + "k", "out_weight": p + "o", "q_norm": p + "q.norm",
                  "k_norm": p + "k.norm"}
         params = {"width": w, "n_head": m.heads, "n_kv_head": m.kv_heads, "head_dim": m.dim, "value_dim": m.vdim,
-                  "scale": m.scale, "rotary": m.rot.part_params(), "qk_norm_eps": eps}
+                  "scale": m.scale, "rotary": m.rot.part_params() if m.rot is not None else None, "qk_norm_eps": eps}
         if kind == "attention":
             names.update(v_weight=p + "v", q_bias=p + "q.b", k_bias=p + "k.b", v_bias=p + "v.b", out_bias=p + "o.b",
                          score_bias=p + "pb")

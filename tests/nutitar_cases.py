@@ -119,7 +119,7 @@ def random_raw(rng) -> dict:
     """A random config.json: two to six layers of random types, widths, head counts and sizes (also no multiples
     of 8), rotations over 2 channels to the whole head, scaled either way or not, windows with and without kept
     tokens or none, latents read by later layers, feed-forwards or none."""
-    width = int(rng.choice([24, 40, 64, 72, 96, 136, 256]))
+    width = int(rng.choice([24, 36, 40, 50, 64, 72, 96, 100, 136, 256]))
 
     def rotation(most, exactly=None):
         dims = exactly or int(rng.choice([d for d in (2, 4, 8, 12, 16, 32, 64, most - most % 2) if 0 < d <= most]))
@@ -140,10 +140,10 @@ def random_raw(rng) -> dict:
     layers, makers = [], []
     for i in range(int(rng.integers(2, 7))):
         pick = rng.random()
-        dim = int(rng.choice([8, 12, 16, 24, 32, 48, 64, 128]))
+        dim = int(rng.choice([6, 8, 10, 12, 16, 24, 32, 48, 64, 128]))
         scale = float(rng.choice([0.1, 0.3, dim ** -0.5]))
         if pick < 0.35:
-            heads, vdim = int(rng.integers(1, 5)), int(rng.choice([8, 16, 20, 32, 64]))
+            heads, vdim = int(rng.integers(1, 5)), int(rng.choice([6, 8, 16, 20, 32, 64]))
             if makers and rng.random() < 0.5:
                 src = int(rng.choice(makers))
                 m = layers[src]["mixer"]
