@@ -32,10 +32,11 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
     float norm_eps, const float* __restrict__ mix_lambda, void* __restrict__ v_other, long ld_other, int mix_mode,
     void* __restrict__ kpool, void* __restrict__ vpool, const int* __restrict__ slot_mapping, int page_size,
     int n_tokens, int norm_mode, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, int v_from_k,
-    float rot_mag) {
+    float rot_mag, int stash) {
   __shared__ float cos_s[QKP_MAX_DIM / 2], sin_s[QKP_MAX_DIM / 2];
   __shared__ float red_s[2 * QKP_MAX_WAVES];
-  extern __shared__ float head_s[];    // [waves][head_dim]: the head a wave is working on
+  extern __shared__ float head_s[];    // [waves][head_dim]: the head a wave is working on; with `stash` behind it
+                                       // [n_head + n_kv_head][head_dim]: the token's queries and keys as loaded
   const int n = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n_waves = blockDim.x >> 6;
   const int half = rot_dims / 2;
@@ -51,14 +52,17 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
   float whole_q = 1.0f, whole_k = 1.0f;   // norm_mode 2: what all query (key) channels of the token are multiplied by
   if (norm_mode == 2) {
     float sq = 0.f, sk = 0.f;
+    float* all_s = head_s + n_waves * head_dim;   // (used with `stash` only)
     for (int i = threadIdx.x; i < n_head * head_dim; i += blockDim.x) {
       const int hh = i / head_dim;
       const float v = load_f(z, dtype, row + q_off + (long)hh * head_stride + (i - hh * head_dim));
+      if (stash) all_s[i] = v;
       sq = fmaf(v, v, sq);
     }
     for (int i = threadIdx.x; i < n_kv_head * head_dim; i += blockDim.x) {
       const int hh = i / head_dim;
       const float v = load_f(z, dtype, row + k_off + (long)hh * head_stride + (i - hh * head_dim));
+      if (stash) all_s[n_head * head_dim + i] = v;
       sk = fmaf(v, v, sk);
     }
     sq = wave_sum(sq);
@@ -86,7 +90,10 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
     const int g = is_q ? hh : hh - n_head;
     if (!is_q && !kpool) continue;
     const long src = row + (is_q ? q_off : k_off) + (long)g * head_stride;
-    for (int c = lane; c < head_dim; c += 64) s[c] = load_f(z, dtype, src + c);
+    if (stash)   // the norm's first pass has the token's queries and keys in LDS already
+      for (int c = lane; c < head_dim; c += 64) s[c] = head_s[(n_waves + hh) * head_dim + c];
+    else
+      for (int c = lane; c < head_dim; c += 64) s[c] = load_f(z, dtype, src + c);
     __builtin_amdgcn_wave_barrier();
     const long dst = ((page * n_kv_head + g) * page_size + off) * (long)head_stride;
     if (v_from_k && !is_q && slot >= 0)   // the values are the keys as projected
@@ -163,11 +170,14 @@ extern "C" int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_of
   if (norm_mode && (!q_norm_w || !k_norm_w)) return MGPT_ERR_NULL;
   // few tokens (a decode step): a wave per head, so that a token's heads are done side by side; many tokens: four
   // waves a token, and more tokens at a time on a compute unit
-  int waves = 4;
-  if (n_tokens < 64 && n_head + n_kv_head > 4) waves = n_head + n_kv_head < QKP_MAX_WAVES ? n_head + n_kv_head : QKP_MAX_WAVES;
-  hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(64 * waves), waves * head_dim * sizeof(float), stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
+  const int heads = n_head + n_kv_head;
+  int waves = heads >= 8 ? 8 : 4;
+  if (n_tokens < 64 && heads > 4) waves = heads < QKP_MAX_WAVES ? heads : QKP_MAX_WAVES;
+  // a norm over the whole projection reads every query and key before any can be normed: they stay in LDS if they fit
+  const int stash = norm_mode == 2 && (size_t)(waves + heads) * head_dim * sizeof(float) <= 48 * 1024;
+  hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(64 * waves), (waves + (stash ? heads : 0)) * head_dim * sizeof(float), stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
                      n_kv_head, head_dim, value_dim, head_stride, positions, rot_dims ? freq : nullptr, rot_dims, norm_eps, mix_lambda,
                      v_other, ld_other, mix_mode, kpool, vpool, slot_mapping, page_size, n_tokens, norm_mode, q_norm_w, k_norm_w,
-                     v_from_k, rot_mag);
+                     v_from_k, rot_mag, stash);
   return mgpt_last_error();
 }
