@@ -68,7 +68,7 @@ extern "C" int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int
   return mgpt_last_error();
 }
 
-#define MAX_DPL 8  // head_dim <= 512
+#define MAX_DPL 16  // head_dim <= 1024
 
 template <typename T, bool FAST_EXP>
 __global__ __launch_bounds__(64) void paged_attention_generic_kernel(

@@ -233,7 +233,7 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
     a visible key's weight is sigmoid(score + score_bias[h]), not normalised over the keys."""
     n_kv_head, page_size, head_dim = _check_attention_args(
         q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
-    _need(head_dim <= 512, f"head size {head_dim} exceeds the kernel's limit of 512")
+    _need(head_dim <= 1024, f"head size {head_dim} exceeds the kernel's limit of 1024")
     _need_sinks(sinks, n_head)
     rc = library.kernels().mgpt_paged_attention_generic(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),

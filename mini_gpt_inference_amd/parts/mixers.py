@@ -186,8 +186,8 @@ class LatentAttention(Mixer):
         # what a cached row holds: the latent alone, or the latent and the rotated key part (rows then
         # start 16 bytes apart in bfloat16 too)
         self.row = self.rank if not self.rot_dim else -(-(self.rank + self.rot_dim) // 8) * 8
-        if not 0 < self.row <= 512:
-            raise ValueError(f"latent size {self.row}: the attention kernels take up to 512")
+        if not 0 < self.row <= 1024:
+            raise ValueError(f"latent size {self.row}: the attention kernels take up to 1024")
         self.q_head = self.head_dim + self.rot_dim
         self.q_width = self.n_head * self.q_head
         self.y_width = self.n_head * self.value_dim
