@@ -83,6 +83,8 @@ int mgpt_linear_mfma(const void* act, long lda, const void* w, const float* bias
     long ldo, int n_rows, int n_out, int k_dim, int epilogue, float* partials, long partials_floats,
     hipStream_t stream);
 // linear_mfma.hip
+int mgpt_linear_mfma_xielu(const void* act, long lda, const void* w, const float* bias, void* out, long ldo,
+    int n_rows, int n_out, int k_dim, const float* coef, float* partials, long partials_floats, hipStream_t stream);
 int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, long lda, const void* w, const float*
     bias, void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue, float* partials,
     long partials_floats, hipStream_t stream);
@@ -232,6 +234,7 @@ int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_st
   X(mgpt_linear_mfma) \
   X(mgpt_linear_mfma_parts) \
   X(mgpt_linear_mfma_shape) \
+  X(mgpt_linear_mfma_xielu) \
   X(mgpt_linear_mfma_qkv) \
   X(mgpt_linear_skinny) \
   X(mgpt_linear_head_best) \

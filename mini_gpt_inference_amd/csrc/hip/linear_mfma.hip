@@ -41,6 +41,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define MM_EPI_GELU 1
 #define MM_EPI_RESIDUAL 2
 #define MM_EPI_QKV 3   // store, and scatter the key and value columns into their cache pages
+#define MM_EPI_XIELU 4 // a_p v^2 + v / 2 for v > 0, a_n (exp(v) - 1 - v) + v / 2 else, (a_p, a_n) from MfmaScatter::epi_coef
+
+__device__ __forceinline__ float mfma_xielu(float v, float a_p, float a_n) {
+  return v > 0.f ? fmaf(a_p * v, v, 0.5f * v) : fmaf(a_n, (__expf(v) - 1.0f) - v, 0.5f * v);
+}
 
 // where the key and value columns of a fused QKV product go (src/minigpt_infer/cache/paged.py:125-137)
 struct MfmaScatter {
@@ -55,6 +60,7 @@ struct MfmaScatter {
   const int* row_valid = nullptr;
   int group_rows = 0;
   long w_stride = 0;
+  const float* epi_coef = nullptr;   // MM_EPI_XIELU: the two coefficients
 };
 
 // The bias of the four neighbouring output columns oc..oc+3 a lane holds.
@@ -76,13 +82,15 @@ __device__ __forceinline__ void mfma_bias4(const float* __restrict__ bias, int o
 // `vec`: the four columns can go as one aligned vector.
 template <int EPI, typename OT>
 __device__ __forceinline__ void mfma_store4(const f32x4_t& a, const float b4[4], OT* __restrict__ out, long ldo,
-                                            int n, int oc, int n_out, bool vec, bf16_t* cache_dst) {
+                                            int n, int oc, int n_out, bool vec, bf16_t* cache_dst, float a_p = 0.f,
+                                            float a_n = 0.f) {
   OT* orow = out + (long)n * ldo;
   float v[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     v[e] = a[e] + b4[e];
     if (EPI == MM_EPI_GELU) v[e] = gelu_tanh_fast(v[e]);
+    if (EPI == MM_EPI_XIELU) v[e] = mfma_xielu(v[e], a_p, a_n);
   }
   if (vec && sizeof(OT) == 4) {
     float4* dst = reinterpret_cast<float4*>(orow + oc);
@@ -422,6 +430,12 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
       }
   }
 
+  // the activation's coefficients, read once (a store in between would make the compiler read them again)
+  float xa_p = 0.f, xa_n = 0.f;
+  if (EPI == MM_EPI_XIELU) {
+    xa_p = sc.epi_coef[0];
+    xa_n = sc.epi_coef[1];
+  }
   // lane holds out[row0 + wr + j*16 + (lane & 15)][col0 + wc + i*16 + (lane >> 4)*4 + e], e = 0..3
   const bool vec = (n_out & 3) == 0 && (ldo & 3) == 0 && (((size_t)out | (size_t)bias) & 15) == 0;
   // bfloat16 outputs go through LDS (the staged operands are done with): a lane's four columns of
@@ -451,6 +465,7 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
             for (int e = 0; e < 4; ++e) {
               v[e] = acc[i][j][e] + b4[e];
               if (EPI == MM_EPI_GELU) v[e] = gelu_tanh_fast(v[e]);
+              if (EPI == MM_EPI_XIELU) v[e] = mfma_xielu(v[e], xa_p, xa_n);
             }
             uint2 pk;
             pk.x = pack_bf16x2(v[0], v[1]);
@@ -517,7 +532,10 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
       if (n >= n_rows) continue;
       bf16_t* cache_dst = nullptr;
       if (EPI == MM_EPI_QKV && cache_col && cache_row[j] >= 0) cache_dst = cache_col + cache_row[j];
-      mfma_store4<EPI, OT>(acc[i][j], b4, out, ldo, n, oc, n_out, vec, cache_dst);
+      if (EPI == MM_EPI_XIELU)
+        mfma_store4<EPI, OT>(acc[i][j], b4, out, ldo, n, oc, n_out, vec, cache_dst, xa_p, xa_n);
+      else
+        mfma_store4<EPI, OT>(acc[i][j], b4, out, ldo, n, oc, n_out, vec, cache_dst);
     }
   }
 }
@@ -555,6 +573,7 @@ int launch_shape(const void* act, long lda, const void* w, const float* bias, vo
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_NONE, bf16_t);
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_NONE, float);
   if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_GELU, bf16_t);
+  if (epilogue == MM_EPI_XIELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_XIELU, bf16_t);
   if (epilogue == MM_EPI_RESIDUAL && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_RESIDUAL, float);
   if (epilogue == MM_EPI_QKV && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_QKV, bf16_t);
 #undef MM_LAUNCH
@@ -662,7 +681,8 @@ int used_parts(int k_dim, int parts) {
 template <int EPI, typename OT>
 __global__ __launch_bounds__(256) void linear_mfma_join_kernel(const float* __restrict__ partials, int k_parts,
                                                                const float* __restrict__ bias, OT* __restrict__ out,
-                                                               long ldo, int n_rows, int n_out) {
+                                                               long ldo, int n_rows, int n_out,
+                                                               const float* __restrict__ epi_coef) {
   const int quads = n_out >> 2;
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (long)n_rows * quads) return;
@@ -686,6 +706,10 @@ __global__ __launch_bounds__(256) void linear_mfma_join_kernel(const float* __re
   if (EPI == MM_EPI_GELU) {
     v.x = gelu_tanh_fast(v.x); v.y = gelu_tanh_fast(v.y); v.z = gelu_tanh_fast(v.z); v.w = gelu_tanh_fast(v.w);
   }
+  if (EPI == MM_EPI_XIELU) {
+    const float a_p = epi_coef[0], a_n = epi_coef[1];
+    v.x = mfma_xielu(v.x, a_p, a_n); v.y = mfma_xielu(v.y, a_p, a_n); v.z = mfma_xielu(v.z, a_p, a_n); v.w = mfma_xielu(v.w, a_p, a_n);
+  }
   OT* orow = out + (long)row * ldo + oc;
   const float r[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -696,15 +720,16 @@ __global__ __launch_bounds__(256) void linear_mfma_join_kernel(const float* __re
 }
 
 int launch_join(const float* partials, int k_parts, const float* bias, void* out, int out_dtype, long ldo,
-                int n_rows, int n_out, int epilogue, hipStream_t stream) {
+                int n_rows, int n_out, int epilogue, hipStream_t stream, const float* epi_coef = nullptr) {
   const long work = (long)n_rows * (n_out >> 2);
   dim3 grid((unsigned int)((work + 255) / 256));
 #define MM_JOIN(E, OT)                                                                                  \
   hipLaunchKernelGGL((linear_mfma_join_kernel<E, OT>), grid, dim3(256), 0, stream, partials, k_parts, \
-                     bias, (OT*)out, ldo, n_rows, n_out)
+                     bias, (OT*)out, ldo, n_rows, n_out, epi_coef)
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_JOIN(MM_EPI_NONE, bf16_t);
   else if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_JOIN(MM_EPI_NONE, float);
   else if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_JOIN(MM_EPI_GELU, bf16_t);
+  else if (epilogue == MM_EPI_XIELU && out_dtype == MGPT_BF16) MM_JOIN(MM_EPI_XIELU, bf16_t);
   else if (epilogue == MM_EPI_RESIDUAL && out_dtype == MGPT_F32) MM_JOIN(MM_EPI_RESIDUAL, float);
   else return MGPT_ERR_BAD_DTYPE;
 #undef MM_JOIN
@@ -875,7 +900,7 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
   }
 #undef MM_ARGS
   if (rc != MGPT_OK || !split || leave_parts) return rc;
-  return launch_join(partials, k_parts, bias, out, out_dtype, ldo, n_rows, n_out, epilogue, stream);
+  return launch_join(partials, k_parts, bias, out, out_dtype, ldo, n_rows, n_out, epilogue, stream, sc.epi_coef);
 }
 
 }  // namespace
@@ -915,6 +940,18 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
   if (epilogue == MM_EPI_QKV) return MGPT_ERR_BAD_SHAPE;  // mgpt_linear_mfma_qkv brings the pools
   MfmaScatter sc = {};
   return launch_any(-1, 0, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, partials,
+                    partials_floats, sc, stream);
+}
+
+// The same product with the xIELU activation behind it (bfloat16 out): coef = float32 (a_p, a_n), the coefficients of
+// v^2 for v > 0 and of (exp(v) - 1 - v) for v <= 0, beside v / 2 in both.
+extern "C" int mgpt_linear_mfma_xielu(const void* act, long lda, const void* w, const float* bias, void* out,
+                                      long ldo, int n_rows, int n_out, int k_dim, const float* coef, float* partials,
+                                      long partials_floats, hipStream_t stream) {
+  if (!coef) return MGPT_ERR_NULL;
+  MfmaScatter sc = {};
+  sc.epi_coef = coef;
+  return launch_any(-1, 0, act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_XIELU, partials,
                     partials_floats, sc, stream);
 }
 

@@ -18,6 +18,7 @@ from . import library
 
 F32, BF16 = 0, 1
 EPI_NONE, EPI_GELU, EPI_RESIDUAL = 0, 1, 2
+EPI_XIELU = 4      # only through linear_mfma_xielu, which brings the activation's coefficients
 
 _ERRORS = {
     -1: "unsupported dtype combination",
@@ -685,6 +686,35 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     if rc == -2:
         return False
     _check(rc, "linear_mfma", 2 if partials is not None else 1)
+    return True
+
+
+def linear_mfma_xielu(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, n_rows: int,
+                      coef: torch.Tensor, partials: Optional[torch.Tensor] = None) -> bool:
+    """The tiled bfloat16 product with the xIELU activation as its epilogue: out = act(a @ w.T (+ bias)) with
+    act(v) = coef[0] v^2 + v / 2 for v > 0 and coef[1] (exp(v) - 1 - v) + v / 2 elsewhere (coef float32 [2]),
+    bfloat16 out.  `partials` as for linear_mfma (linear_mfma_partials with EPI_XIELU says how much).  False when
+    it does not take the shape."""
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        return False
+    n_out, k_dim = w.shape
+    if k_dim % 16 != 0 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0 or w.data_ptr() % 16 != 0:
+        return False
+    _need_cuda(a, w, bias, out, coef, partials)
+    _need(w.is_contiguous(), "weight must be dense [out, in]")
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_rows,
+          "activation must be [>=n_rows, inner] with unit inner stride")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_out and out.shape[0] >= n_rows,
+          "output must be [>=n_rows, >=out] with unit inner stride")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
+    _need(coef.dtype == torch.float32 and coef.is_contiguous() and coef.numel() == 2, "coef must be float32 [2]")
+    _need(partials is None or (partials.dtype == torch.float32 and partials.is_contiguous()), "partials must be dense float32")
+    rc = library.kernels().mgpt_linear_mfma_xielu(
+        _ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out), out.stride(0), n_rows, n_out, k_dim, _ptr(coef),
+        _ptr(partials), 0 if partials is None else partials.numel(), _stream())
+    if rc == -2:
+        return False
+    _check(rc, "linear_mfma_xielu", 2 if partials is not None else 1)
     return True
 
 

@@ -131,6 +131,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P, L, I, P, P],
         "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P, F, P, L, I, P, P],
         "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P, L, P],
+        "mgpt_linear_mfma_xielu": [P, L, P, P, P, L, I, I, I, P, P, L, P],
         "mgpt_linear_mfma_shape": [I, I, P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_partials": [I, I, I, I],
         "mgpt_linear_mfma_parts": [P, L, P, P, P, L, I, I, I, P],

@@ -250,6 +250,27 @@ def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
     linear(ctx, a, w, bias, x, n_rows, kernels.EPI_RESIDUAL)
 
 
+def linear_xielu(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                 n_rows: int, coef: torch.Tensor) -> None:
+    """out[:n_rows] = xielu(a[:n_rows] @ w.T (+ bias)) with the activation's two coefficients in `coef` (float32
+    [2]).  Where the product goes to the tiled MFMA kernel (steps of many rows, and few rows under a large matrix)
+    the activation is that kernel's epilogue; everywhere else (the decode kernel, the 32-bit path) it is a kernel of
+    its own behind the product, in place."""
+    if n_rows == 0:
+        return
+    fast = (w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16 and w.shape[1] % 16 == 0
+            and out.dtype == torch.bfloat16)
+    wide_out = w.shape[0] >= WIDE_OUT and n_rows * w.shape[1] > WIDE_OUT_DECODE_WORK
+    if fast and not (n_rows <= 64 and not wide_out and not tiled_at_few_rows(n_rows, w)):
+        a = as_tensor(ctx, a)
+        need = kernels.linear_mfma_partials(n_rows, w.shape[0], w.shape[1], kernels.EPI_XIELU)
+        partials = ctx.workspace.get("linear_partials", need, 1, torch.float32) if need else None
+        if kernels.linear_mfma_xielu(a, w, bias, out, n_rows, coef, partials=partials):
+            return
+    linear(ctx, a, w, bias, out, n_rows)
+    kernels.xielu(out, out, coef, n_rows, w.shape[0], fast=not ctx.exact)
+
+
 def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optional[torch.Tensor],
            out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None,
            tile_best: Optional[TileBest] = None) -> bool:

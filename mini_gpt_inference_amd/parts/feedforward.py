@@ -7,10 +7,11 @@ from typing import Dict
 import torch
 
 from ..ops import kernels, residual
-from ..ops.linear import LazyNorm, as_tensor, linear, linear_add, packed_weight, plain_residual
+from ..ops.linear import LazyNorm, as_tensor, linear, linear_add, linear_xielu, packed_weight, plain_residual
 from .base import MATRIX, Part, StepContext, TABLE, VECTOR, WeightRequest, register_feed_forward
 
-# activations of the dense feed-forward: an epilogue of the product kernels, or (None) a kernel of its own behind them
+# activations of the dense feed-forward: an epilogue of the product kernels, or (None) one that brings coefficients
+# (ops.linear.linear_xielu: the tiled kernel's epilogue, elsewhere a kernel of its own behind the product)
 _ACTIVATIONS = {"gelu_tanh": kernels.EPI_GELU, "xielu": None}
 
 
@@ -90,10 +91,10 @@ class DenseMLP(FeedForward):
         plain_residual(ctx, h, x)
         n = ctx.n_rows
         u = ctx.workspace.get("ff_hidden", n, self.hidden, ctx.dtype)
-        epilogue = _ACTIVATIONS[self.activation]
-        linear(ctx, h, self.fc_weight, self.fc_bias, u, n, kernels.EPI_NONE if epilogue is None else epilogue)
         if self.activation == "xielu":
-            kernels.xielu(u, u, self.act_coef, n, self.hidden, fast=not ctx.exact)
+            linear_xielu(ctx, h, self.fc_weight, self.fc_bias, u, n, self.act_coef)
+        else:
+            linear(ctx, h, self.fc_weight, self.fc_bias, u, n, _ACTIVATIONS[self.activation])
         # (a caller that hands over a LazyNorm of x itself knows that x may be left as a sum)
         linear_add(ctx, u, self.proj_weight, self.proj_bias, x, n,
                    may_leave_parts=isinstance(h, LazyNorm) and h.x is x)

@@ -78,6 +78,25 @@ def test_xielu(dtype, n, hidden):
         assert (out[:, hidden:] == 9.0).all()
 
 
+@pytest.mark.parametrize("n,k,out,bias", [(300, 256, 1000, True), (8, 2048, 8192, False), (64, 4096, 256, False),
+                                          (2048, 512, 2048, True), (33, 64, 72, False)])
+def test_xielu_as_the_tiled_products_epilogue(n, k, out, bias):
+    """The activation inside the tiled bfloat16 product, also where the inner size is split among workgroups and
+    the parts are joined by a second kernel."""
+    g = torch.Generator().manual_seed(n + k + out)
+    a, w = _rnd(g, n, k, dtype="bfloat16"), _rnd(g, out, k, dtype="bfloat16", scale=k ** -0.5)
+    b = _rnd(g, out, scale=0.3) if bias else None
+    p, q = torch.tensor(-0.2), torch.tensor(0.6)
+    want = P.xielu(_d(a) @ _d(w).T + (_d(b) if bias else 0.0), _d(p), _d(q))
+    coef = torch.stack([torch.nn.functional.softplus(p), torch.nn.functional.softplus(q) + 0.5]).to(DEV)
+    need = kernels.linear_mfma_partials(n, out, k, kernels.EPI_XIELU)
+    partials = torch.empty(need, dtype=torch.float32, device=DEV) if need else None
+    got = torch.full((n, out + 8), 9.0, dtype=torch.bfloat16, device=DEV)
+    assert kernels.linear_mfma_xielu(a.to(DEV), w.to(DEV), b.to(DEV) if bias else None, got, n, coef, partials=partials)
+    helpers.assert_close(got[:, :out], want, "bfloat16", f"xielu epilogue, {'split' if need else 'whole'} inner size")
+    assert (got[:, out:] == 9.0).all()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("width,pad", [(40, 3), (40, 0), (256, 4), (1030, 2), (2048, 0), (3076, 8)])
 def test_norm_and_token_shift_keep_a_row_per_request(dtype, width, pad):
