@@ -29,7 +29,8 @@ def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, w
             return True
         # the decode kernel refuses this head or page size: the tile kernel for the leading requests too
         return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
-                                              lead, 1, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate, **mask)
+                                              lead, 1, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate,
+                                              **mask)
     return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                           ctx.n_req, ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap,
                                           gate=gate, **mask)
@@ -77,8 +78,8 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
         if not ctx.decode_only and not ctx.padded and _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head, scale,
                                                                   window, sinks, softcap, gate, keep_first, score_bias):
             return
-        if not ctx.decode_only and ctx.padded and _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head,
-                                                                     scale, window, sinks, softcap, gate, keep_first, score_bias):
+        if not ctx.decode_only and ctx.padded and _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head, scale,
+                                                                     window, sinks, softcap, gate, keep_first, score_bias):
             return
         if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                               ctx.q_req, n, r, n_head, scale, window, sinks=sinks, softcap=softcap,
