@@ -164,9 +164,9 @@ def config_from_json(raw: Mapping[str, Any]) -> NutitarConfig:
         if mixer.kv_from is not None:
             src = layers[mixer.kv_from] if mixer.kv_from < i else None
             if (src is None or src.type != "latent_attention" or src.mixer.kv_from is not None
-                    or (src.mixer.kv_rank, src.mixer.rot_dim, src.mixer.rot) != (mixer.kv_rank, mixer.rot_dim, mixer.rot)):
+                    or (src.mixer.kv_rank, src.mixer.rot_dim) != (mixer.kv_rank, mixer.rot_dim)):
                 raise ConfigError(f"layer {i}: kv_from names an earlier latent-attention layer that makes its own "
-                                  f"latents, with this layer's kv_rank, rot_dim and rot")
+                                  f"latents, with this layer's kv_rank and rot_dim")
         mlp = layer.get("mlp")
         if mlp is not None and mlp.get("kind") != "dense":
             raise ConfigError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")

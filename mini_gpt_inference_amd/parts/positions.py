@@ -96,8 +96,6 @@ class RotaryHalf(PositionEncoding):
                 raise ValueError(f"rotation scaling {scaling!r}: kind 'stretch' or 'ramp' with {wanted}")
             if not float(self.scaling["factor"]) > 0.0 or not float(self.scaling["original"]) > 0.0:
                 raise ValueError("rotation scaling: factor and original must be positive")
-            if kind == "stretch" and float(self.scaling["high"]) == float(self.scaling["low"]):
-                raise ValueError("rotation scaling: low and high must differ")
             if kind == "ramp":
                 if not (float(self.scaling["fast"]) > 0.0 and float(self.scaling["slow"]) > 0.0) or self.base == 1.0:
                     raise ValueError("rotation scaling: fast and slow must be positive, and the base not 1")
@@ -118,6 +116,8 @@ class RotaryHalf(PositionEncoding):
                 if wavelength < original / high:
                     out.append(f)
                 elif wavelength > original / low:
+                    out.append(f / factor)
+                elif high == low:      # (no wavelength lies between two equal bounds; one that sits on them counts as long)
                     out.append(f / factor)
                 else:
                     s = (original / wavelength - low) / (high - low)
