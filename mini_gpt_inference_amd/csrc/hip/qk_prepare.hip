@@ -23,14 +23,19 @@
 #include "dtype_io.h"
 #include "launchers.h"
 
+template <typename T> __device__ __forceinline__ float qk_load(const T* p, long i) { return to_float<T>(p[i]); }
+template <typename T> __device__ __forceinline__ void qk_store(T* p, long i, float v) { p[i] = from_float<T>(v); }
+
 #define QKP_MAX_DIM 512
 #define QKP_MAX_WAVES 16   // a wave a head at a time: as many waves as the token has query and key heads, up to these
 
+// T: the storage type of z, the pools and v_other (a type known at compile time lets a lane's loads be in flight together)
+template <typename T>
 __global__ __launch_bounds__(1024) void qk_prepare_kernel(
-    void* __restrict__ z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head, int n_kv_head,
+    T* __restrict__ z, long ldz, int q_off, int k_off, int v_off, int n_head, int n_kv_head,
     int head_dim, int value_dim, int head_stride, const int* __restrict__ positions, const float* __restrict__ freq, int rot_dims,
-    float norm_eps, const float* __restrict__ mix_lambda, void* __restrict__ v_other, long ld_other, int mix_mode,
-    void* __restrict__ kpool, void* __restrict__ vpool, const int* __restrict__ slot_mapping, int page_size,
+    float norm_eps, const float* __restrict__ mix_lambda, T* __restrict__ v_other, long ld_other, int mix_mode,
+    T* __restrict__ kpool, T* __restrict__ vpool, const int* __restrict__ slot_mapping, int page_size,
     int n_tokens, int norm_mode, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, int v_from_k,
     float rot_mag, int stash) {
   __shared__ float cos_s[QKP_MAX_DIM / 2], sin_s[QKP_MAX_DIM / 2];
@@ -55,13 +60,13 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
     float* all_s = head_s + n_waves * head_dim;   // (used with `stash` only)
     for (int i = threadIdx.x; i < n_head * head_dim; i += blockDim.x) {
       const int hh = i / head_dim;
-      const float v = load_f(z, dtype, row + q_off + (long)hh * head_stride + (i - hh * head_dim));
+      const float v = qk_load<T>(z, row + q_off + (long)hh * head_stride + (i - hh * head_dim));
       if (stash) all_s[i] = v;
       sq = fmaf(v, v, sq);
     }
     for (int i = threadIdx.x; i < n_kv_head * head_dim; i += blockDim.x) {
       const int hh = i / head_dim;
-      const float v = load_f(z, dtype, row + k_off + (long)hh * head_stride + (i - hh * head_dim));
+      const float v = qk_load<T>(z, row + k_off + (long)hh * head_stride + (i - hh * head_dim));
       if (stash) all_s[n_head * head_dim + i] = v;
       sk = fmaf(v, v, sk);
     }
@@ -93,11 +98,11 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
     if (stash)   // the norm's first pass has the token's queries and keys in LDS already
       for (int c = lane; c < head_dim; c += 64) s[c] = head_s[(n_waves + hh) * head_dim + c];
     else
-      for (int c = lane; c < head_dim; c += 64) s[c] = load_f(z, dtype, src + c);
+      for (int c = lane; c < head_dim; c += 64) s[c] = qk_load<T>(z, src + c);
     __builtin_amdgcn_wave_barrier();
     const long dst = ((page * n_kv_head + g) * page_size + off) * (long)head_stride;
     if (v_from_k && !is_q && slot >= 0)   // the values are the keys as projected
-      for (int c = lane; c < head_stride; c += 64) store_f(vpool, dtype, dst + c, c < head_dim ? s[c] : 0.f);
+      for (int c = lane; c < head_stride; c += 64) qk_store<T>(vpool, dst + c, c < head_dim ? s[c] : 0.f);
     if (norm_mode == 1) {
       float ss = 0.f;
       for (int c = lane; c < head_dim; c += 64) ss = fmaf(s[c], s[c], ss);
@@ -126,9 +131,9 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
       r = 1.0f / sqrtf(wave_sum(ss) / (float)head_dim + norm_eps);
     }
     if (is_q) {
-      for (int c = lane; c < head_dim; c += 64) store_f(z, dtype, src + c, s[c] * r);
+      for (int c = lane; c < head_dim; c += 64) qk_store<T>(z, src + c, s[c] * r);
     } else if (slot >= 0) {
-      for (int c = lane; c < head_stride; c += 64) store_f(kpool, dtype, dst + c, c < head_dim ? s[c] * r : 0.f);
+      for (int c = lane; c < head_stride; c += 64) qk_store<T>(kpool, dst + c, c < head_dim ? s[c] * r : 0.f);
       if (v_from_k) {
         __builtin_amdgcn_wave_barrier();
         continue;
@@ -137,16 +142,16 @@ __global__ __launch_bounds__(1024) void qk_prepare_kernel(
       const long osrc = (long)n * ld_other + (long)g * value_dim;
       const float lam = mix_mode == 2 ? mix_lambda[0] : 0.f;
       for (int c = lane; c < head_stride; c += 64) {
-        float v = load_f(z, dtype, vsrc + c);
-        if (mix_mode == 1 && c < value_dim) store_f(v_other, dtype, osrc + c, v);
-        if (mix_mode == 2 && c < value_dim) v = (1.0f - lam) * v + lam * load_f(v_other, dtype, osrc + c);
-        store_f(vpool, dtype, dst + c, v);
+        float v = qk_load<T>(z, vsrc + c);
+        if (mix_mode == 1 && c < value_dim) qk_store<T>(v_other, osrc + c, v);
+        if (mix_mode == 2 && c < value_dim) v = (1.0f - lam) * v + lam * qk_load<T>(v_other, osrc + c);
+        qk_store<T>(vpool, dst + c, v);
       }
     } else if (mix_mode == 1) {
       // a token without a slot (padding of a bucket) still leaves its values: rows are independent
       const long vsrc = row + v_off + (long)g * head_stride;
       const long osrc = (long)n * ld_other + (long)g * value_dim;
-      for (int c = lane; c < value_dim; c += 64) store_f(v_other, dtype, osrc + c, load_f(z, dtype, vsrc + c));
+      for (int c = lane; c < value_dim; c += 64) qk_store<T>(v_other, osrc + c, qk_load<T>(z, vsrc + c));
     }
     __builtin_amdgcn_wave_barrier();
   }
@@ -175,9 +180,13 @@ extern "C" int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_of
   if (n_tokens < 64 && heads > 4) waves = heads < QKP_MAX_WAVES ? heads : QKP_MAX_WAVES;
   // a norm over the whole projection reads every query and key before any can be normed: they stay in LDS if they fit
   const int stash = norm_mode == 2 && (size_t)(waves + heads) * head_dim * sizeof(float) <= 48 * 1024;
-  hipLaunchKernelGGL(qk_prepare_kernel, dim3(n_tokens), dim3(64 * waves), (waves + (stash ? heads : 0)) * head_dim * sizeof(float), stream, z, dtype, ldz, q_off, k_off, v_off, n_head,
-                     n_kv_head, head_dim, value_dim, head_stride, positions, rot_dims ? freq : nullptr, rot_dims, norm_eps, mix_lambda,
-                     v_other, ld_other, mix_mode, kpool, vpool, slot_mapping, page_size, n_tokens, norm_mode, q_norm_w, k_norm_w,
-                     v_from_k, rot_mag, stash);
+#define QKP_LAUNCH(T)                                                                                                  \
+  hipLaunchKernelGGL(qk_prepare_kernel<T>, dim3(n_tokens), dim3(64 * waves), (waves + (stash ? heads : 0)) * head_dim * sizeof(float), \
+                     stream, (T*)z, ldz, q_off, k_off, v_off, n_head, n_kv_head, head_dim, value_dim, head_stride, positions,  \
+                     rot_dims ? freq : nullptr, rot_dims, norm_eps, mix_lambda, (T*)v_other, ld_other, mix_mode, (T*)kpool,    \
+                     (T*)vpool, slot_mapping, page_size, n_tokens, norm_mode, q_norm_w, k_norm_w, v_from_k, rot_mag, stash)
+  if (dtype == MGPT_F32) QKP_LAUNCH(float);
+  else QKP_LAUNCH(bf16_t);
+#undef QKP_LAUNCH
   return mgpt_last_error();
 }
